@@ -37,13 +37,17 @@ def k_page_elems(req: PagedKv, page_size: int) -> int:
     return req.n_kv_heads * req.head_dim * page_size
 
 
+def v_page_elems(req: PagedKv, page_size: int) -> int:
+    return req.n_kv_heads * req.v_dim * page_size
+
+
 class PagedGroup:
     """Cache units with one requirement: a pool, a block table per slot, and the page tensors.
 
     Device layout of one unit: keys ``[page, kv_head, head_dim/8, page_size, 8]`` (a run of 8
     consecutive head dimensions of one token is contiguous, tokens of a page next to each
-    other), values ``[page, kv_head, head_dim, page_size]`` (transposed: the tokens of a page
-    are contiguous for one head dimension). Both are what the matrix instructions of the
+    other), values ``[page, kv_head, value_dim, page_size]`` (transposed: the tokens of a page
+    are contiguous for one dimension; ``value_dim`` is ``head_dim`` unless the requirement says otherwise). Both are what the matrix instructions of the
     attention kernels read without a transposition."""
 
     def __init__(self, index: int, req: PagedKv, units: List[int], n_pages: int, page_size: int, max_seqs: int,
@@ -61,13 +65,13 @@ class PagedGroup:
         self.unit_pos = {u: i for i, u in enumerate(self.units)}
 
     def allocate_tensors(self, dtype: torch.dtype, device) -> None:
-        elems = k_page_elems(self.requirement, self.page_size)
-        shape = (len(self.units), self.pool.n_pages, elems)
-        self.k_pages = torch.zeros(shape, dtype=dtype, device=device)
-        self.v_pages = torch.zeros(shape, dtype=dtype, device=device)
+        n = (len(self.units), self.pool.n_pages)
+        self.k_pages = torch.zeros(n + (k_page_elems(self.requirement, self.page_size),), dtype=dtype, device=device)
+        self.v_pages = torch.zeros(n + (v_page_elems(self.requirement, self.page_size),), dtype=dtype, device=device)
 
     def bytes_per_token(self, itemsize: int) -> int:
-        return 2 * len(self.units) * self.requirement.n_kv_heads * self.requirement.head_dim * itemsize
+        r = self.requirement
+        return len(self.units) * r.n_kv_heads * (r.head_dim + r.v_dim) * itemsize
 
     # ---- per-request bookkeeping -------------------------------------------------
     def blocks_needed(self, slot: int, old_len: int, new_len: int) -> int:

@@ -13,6 +13,11 @@ class PagedKv:
     n_kv_heads: int
     head_dim: int
     window: Optional[int] = None  # None: all keys. w: a query at position p reads keys p-w+1 .. p
+    value_dim: Optional[int] = None  # size of a value head where it differs from a key head's (None: head_dim)
+
+    @property
+    def v_dim(self) -> int:
+        return self.head_dim if self.value_dim is None else self.value_dim
 
 
 @dataclass(frozen=True)

@@ -20,7 +20,7 @@ GIB = 1 << 30
 
 def group_page_bytes(req: PagedKv, n_units: int, page_size: int, itemsize: int) -> int:
     """Bytes of one page of a group: keys and values of ``page_size`` tokens in each of its cache units."""
-    return 2 * n_units * req.n_kv_heads * req.head_dim * page_size * itemsize
+    return n_units * req.n_kv_heads * (req.head_dim + req.v_dim) * page_size * itemsize
 
 
 def window_group_pages(req: PagedKv, page_size: int, max_seqs: int, max_pages_per_seq: int, longest_portion: int) -> int:

@@ -1,5 +1,6 @@
 from .lm_config import ConfigError, LmConfig
 from .gpt2 import Gpt2Config
+from .zederax import ZederaxConfig
 from .engine_config import InferenceEngineConfig
 
-__all__ = ["ConfigError", "LmConfig", "Gpt2Config", "InferenceEngineConfig"]
+__all__ = ["ConfigError", "LmConfig", "Gpt2Config", "ZederaxConfig", "InferenceEngineConfig"]

@@ -4,7 +4,7 @@ The reference keeps a plugin registry on ``LmConfig`` (src/levanter/models/lm_mo
 that maps a name such as ``"gpt2"`` to a config class, and each config class knows its model
 (``model_type``, src/levanter/models/gpt2.py:74-76) and how to read a checkpoint's
 ``config.json`` (``from_hf_config``, gpt2.py:102-117). Here the registry key is the
-``model_type`` field of ``config.json``.
+``model_type`` field of ``config.json`` or, in files without one, their ``architecture`` in lower case.
 """
 from __future__ import annotations
 
@@ -81,9 +81,13 @@ class LmConfig:
 
     @staticmethod
     def from_dict(raw: Dict[str, Any]) -> "LmConfig":
-        if "model_type" not in raw:
-            raise ConfigError("config.json has no 'model_type' key")
-        return LmConfig.get_choice_class(raw["model_type"]).from_hf_config(raw)
+        # the architecture's name: ``model_type``, or (files that have no such key) ``architecture``, in any case
+        name = raw.get("model_type")
+        if name is None and isinstance(raw.get("architecture"), str):
+            name = raw["architecture"].lower()
+        if name is None:
+            raise ConfigError("config.json has neither a 'model_type' nor an 'architecture' key")
+        return LmConfig.get_choice_class(name).from_hf_config(raw)
 
     def save(self, model_dir: str) -> None:
         os.makedirs(model_dir, exist_ok=True)

@@ -261,17 +261,17 @@ __device__ __forceinline__ void copy8(T* dst, const T* src) {  // 8 elements, bo
 template <typename T>
 __global__ void kv_write_kernel(const T* __restrict__ k, const T* __restrict__ v, long k_stride, long v_stride,
                                 T* __restrict__ k_pages, T* __restrict__ v_pages, const int* __restrict__ dest, int n_tokens,
-                                int KVH, int HD, int PS, int vec_ok) {
+                                int KVH, int HD, int VD, int PS, int vec_ok) {
   extern __shared__ __attribute__((aligned(16))) unsigned char kvw_smem[];
   int* dst_s = reinterpret_cast<int*>(kvw_smem);                       // [KVW_TOKENS]
-  T* vt = reinterpret_cast<T*>(kvw_smem + KVW_TOKENS * sizeof(int));   // [KVW_TOKENS][HD + 8]
-  const int ldv = HD + 8;
+  T* vt = reinterpret_cast<T*>(kvw_smem + KVW_TOKENS * sizeof(int));   // [KVW_TOKENS][VD + 8]
+  const int ldv = VD + 8;
   const int t0 = blockIdx.x * KVW_TOKENS;
   const int h = blockIdx.y;
   const int tid = threadIdx.x;
   if (tid < KVW_TOKENS) dst_s[tid] = t0 + tid < n_tokens ? dest[t0 + tid] : -1;
-  const int chunks = HD / 8;
-  // keys: one chunk of one token per thread and turn; values into LDS on the way
+  const int chunks = HD / 8, v_chunks = VD / 8;
+  // keys: one chunk of one token per thread and turn
   for (int idx = tid; idx < KVW_TOKENS * chunks; idx += blockDim.x) {
     const int i = idx / chunks, c = idx % chunks;
     const int t = t0 + i;
@@ -279,22 +279,31 @@ __global__ void kv_write_kernel(const T* __restrict__ k, const T* __restrict__ v
     const int dst = dest[t];
     if (dst < 0) continue;
     const T* kr = k + (size_t)t * k_stride + (size_t)h * HD + c * 8;
-    const T* vr = v + (size_t)t * v_stride + (size_t)h * HD + c * 8;
     const int page = dst / PS, off = dst % PS;
     T* kd = k_pages + ((size_t)page * KVH + h) * (size_t)HD * PS + ((size_t)c * PS + off) * 8;
     if (vec_ok) {
       copy8<T>(kd, kr);
+    } else {
+#pragma unroll
+      for (int e = 0; e < 8; ++e) kd[e] = kr[e];
+    }
+  }
+  // values into LDS on the way (a value head may have another size than a key head)
+  for (int idx = tid; idx < KVW_TOKENS * v_chunks; idx += blockDim.x) {
+    const int i = idx / v_chunks, c = idx % v_chunks;
+    const int t = t0 + i;
+    if (t >= n_tokens) continue;
+    if (dest[t] < 0) continue;
+    const T* vr = v + (size_t)t * v_stride + (size_t)h * VD + c * 8;
+    if (vec_ok) {
       copy8<T>(vt + i * ldv + c * 8, vr);
     } else {
 #pragma unroll
-      for (int e = 0; e < 8; ++e) {
-        kd[e] = kr[e];
-        vt[i * ldv + c * 8 + e] = vr[e];
-      }
+      for (int e = 0; e < 8; ++e) vt[i * ldv + c * 8 + e] = vr[e];
     }
   }
   __syncthreads();
-  for (int d = tid; d < HD; d += blockDim.x) {
+  for (int d = tid; d < VD; d += blockDim.x) {
     int i = 0;
     while (i < KVW_TOKENS) {
       const int dst = dst_s[i];
@@ -303,7 +312,7 @@ __global__ void kv_write_kernel(const T* __restrict__ k, const T* __restrict__ v
         continue;
       }
       const int page = dst / PS, off = dst % PS;
-      T* vd = v_pages + ((size_t)page * KVH + h) * (size_t)HD * PS + (size_t)d * PS + off;
+      T* vd = v_pages + ((size_t)page * KVH + h) * (size_t)VD * PS + (size_t)d * PS + off;
       bool run = vec_ok && (off % 8 == 0) && i + 8 <= KVW_TOKENS;
       if (run) {
 #pragma unroll
@@ -323,28 +332,30 @@ __global__ void kv_write_kernel(const T* __restrict__ k, const T* __restrict__ v
   }
 }
 
+// HD: elements of a key head, VD: of a value head (the two differ in some architectures)
 extern "C" int lev_kv_write(const void* k, const void* v, long k_stride, long v_stride, void* k_pages, void* v_pages,
-                            const int* dest, int T, int KVH, int HD, int PS, int dtype, hipStream_t stream) {
+                            const int* dest, int T, int KVH, int HD, int VD, int PS, int dtype, hipStream_t stream) {
   LEV_REQUIRE(T >= 0 && KVH > 0, "kv_write: bad sizes T=%d kv_heads=%d", T, KVH);
-  LEV_REQUIRE(HD > 0 && HD % 8 == 0, "kv_write: head_dim=%d must be a multiple of 8", HD);
+  LEV_REQUIRE(HD > 0 && HD % 8 == 0 && VD > 0 && VD % 8 == 0, "kv_write: head sizes %d (keys) and %d (values) must be multiples of 8", HD, VD);
   LEV_REQUIRE(PS > 0 && PS % 16 == 0, "kv_write: page_size=%d must be a multiple of 16", PS);
   LEV_REQUIRE(KVH <= 65535, "kv_write: too many kv heads (%d)", KVH);
   LEV_REQUIRE(dtype == LEV_F32 || dtype == LEV_BF16, "kv_write: unknown dtype %d", dtype);
   if (T == 0) return 0;
   const size_t esize = dtype == LEV_F32 ? 4 : 2;
-  const size_t lds = KVW_TOKENS * sizeof(int) + (size_t)KVW_TOKENS * (HD + 8) * esize;
-  LEV_REQUIRE(lds <= 64 * 1024, "kv_write: head_dim=%d is too large", HD);
-  // 16-byte copies of the source rows need aligned rows (the pages always are: page_size and head_dim are multiples of 8)
+  const size_t lds = KVW_TOKENS * sizeof(int) + (size_t)KVW_TOKENS * (VD + 8) * esize;
+  LEV_REQUIRE(lds <= 64 * 1024, "kv_write: a value head of %d is too large", VD);
+  // 16-byte copies of the source rows need aligned rows (the pages always are: page_size and head sizes are multiples of 8)
   const int vec_ok = ((uintptr_t)k % 16 == 0) && ((uintptr_t)v % 16 == 0) && (k_stride * esize % 16 == 0) && (v_stride * esize % 16 == 0) &&
                      ((uintptr_t)k_pages % 16 == 0) && ((uintptr_t)v_pages % 16 == 0);
   dim3 grid((T + KVW_TOKENS - 1) / KVW_TOKENS, KVH);
-  const int nt = HD <= 64 ? 64 : (HD <= 128 ? 128 : 256);
+  const int widest = HD > VD ? HD : VD;
+  const int nt = widest <= 64 ? 64 : (widest <= 128 ? 128 : 256);
   if (dtype == LEV_F32)
     kv_write_kernel<float><<<grid, nt, lds, stream>>>((const float*)k, (const float*)v, k_stride, v_stride, (float*)k_pages,
-                                                      (float*)v_pages, dest, T, KVH, HD, PS, vec_ok);
+                                                      (float*)v_pages, dest, T, KVH, HD, VD, PS, vec_ok);
   else
     kv_write_kernel<bf16_t><<<grid, nt, lds, stream>>>((const bf16_t*)k, (const bf16_t*)v, k_stride, v_stride,
-                                                       (bf16_t*)k_pages, (bf16_t*)v_pages, dest, T, KVH, HD, PS, vec_ok);
+                                                       (bf16_t*)k_pages, (bf16_t*)v_pages, dest, T, KVH, HD, VD, PS, vec_ok);
   return lev_check_launch("kv_write");
 }
 

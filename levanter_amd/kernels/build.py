@@ -1,6 +1,7 @@
 """Compiles the HIP sources under ``csrc/`` into shared libraries for gfx950, one per unit:
 
-* ``core``: errors, embedding / norms / KV write / sampling, the 32-bit GEMM and attention;
+* ``core``: errors, embedding / norms / KV write / sampling, the row-wise steps of other layer designs, the 32-bit GEMM and
+  the 32-bit attentions;
 * ``gemm_mfma``: the bfloat16 GEMMs on the matrix cores;
 * ``gemm_library``: the vendor library's GEMM (hipBLASLt) for prompt-sized row counts, where it is ahead;
 * ``attn_hd<N>``: the bfloat16 attention on the matrix cores for head size N (16 .. 128 in steps of 16).
@@ -254,11 +255,17 @@ def ensure_built(unit: str = "core") -> str:
 # ---- the units of this package --------------------------------------------------------------------------------
 _P, _I, _L, _F = ctypes.c_void_p, ctypes.c_int, ctypes.c_long, ctypes.c_float
 
-register_unit("core", ["errors.hip", "elementwise.hip", "gemm_simple.hip", "attention_simple.hip", "attention_common.hip"], signatures={
+register_unit("core", ["errors.hip", "elementwise.hip", "layer_ops.hip", "gemm_simple.hip", "attention_simple.hip", "attention_values.hip",
+                       "attention_common.hip"], signatures={
     "lev_embed": [_P] * 5 + [_I, _I, _I, _P],
     "lev_norm": [_P] * 5 + [_I, _I, _F, _I, _I, _P],
     "lev_norm_pending": [_P, _P, _I] + [_P] * 5 + [_I, _I, _I, _F, _I, _I, _P],
-    "lev_kv_write": [_P, _P, _L, _L, _P, _P, _P] + [_I] * 5 + [_P],
+    "lev_kv_write": [_P, _P, _L, _L, _P, _P, _P] + [_I] * 6 + [_P],
+    "lev_head_prepare": [_P, _L, _I, _I, _F, _P, _L, _P, _L, _I, _I, _P, _I, _I, _P],
+    "lev_poly_norm": [_P, _L, _P, _L, _P, _I, _I, _F, _I, _P],
+    "lev_head_talk": [_P, _P, _P, _L, _P, _L] + [_I] * 6 + [_P],
+    "lev_stream_average": [_P, _P, _P, _I, _L, _P],
+    "lev_attention_values": [_P, _L, _P, _P, _P, _P, _P, _P] + [_I] * 8 + [_F, _I, _F, _P, _I, _P],
     "lev_sample": [_P, _L, _P, _P, _P, _P, _P, _P, _I, _I, _P],
     "lev_sample_workspace": [_I],
     "lev_feed_tokens": [_P, _P, _P, _I, _P],

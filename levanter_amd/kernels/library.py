@@ -334,23 +334,108 @@ class HipKernels:
         return not (K >= 4 * N and M < 1024)
 
     # ---- cache write -----------------------------------------------------------------------
-    def kv_write(self, k, v, k_pages, v_pages, dest, n_kv_heads: int, head_dim: int, page_size: int) -> None:
-        """Scatter the new tokens' keys and values ([T, n_kv_heads*head_dim] views) to ``dest[t] = page*page_size + offset``."""
+    def kv_write(self, k, v, k_pages, v_pages, dest, n_kv_heads: int, head_dim: int, page_size: int, value_dim: Optional[int] = None) -> None:
+        """Scatter the new tokens' keys and values ([T, n_kv_heads*head_dim] views; values [T, n_kv_heads*value_dim] where a
+        value head has a size of its own) to ``dest[t] = page*page_size + offset``."""
         if not (k.is_cuda and v.is_cuda and k_pages.is_cuda and v_pages.is_cuda and dest.is_cuda):
             raise KernelError("a kernel was given a tensor that is not on the GPU")
         T, cols = k.shape
         dt = k.dtype
-        if not (v.shape == k.shape and cols == n_kv_heads * head_dim):
-            raise KernelError("kv_write: k and v must be [T, kv_heads*head_dim]")
+        vd = head_dim if value_dim is None else int(value_dim)
+        if not (v.shape == (T, n_kv_heads * vd) and cols == n_kv_heads * head_dim):
+            raise KernelError("kv_write: k must be [T, kv_heads*head_dim] and v [T, kv_heads*value_dim]")
         if not (dt == v.dtype == k_pages.dtype == v_pages.dtype and dt in _DT):
             raise KernelError("kv_write: dtypes differ")
         if not (dest.dtype == torch.int32 and dest.numel() == T):
             raise KernelError("kv_write: one int32 destination per token")
         n_elems = k_pages.numel()
-        if not (k_pages.is_contiguous() and v_pages.is_contiguous() and n_elems % (cols * page_size) == 0 and n_elems == v_pages.numel()):
+        if not (k_pages.is_contiguous() and v_pages.is_contiguous() and n_elems % (cols * page_size) == 0
+                and n_elems * vd == v_pages.numel() * head_dim):
             raise KernelError("kv_write: page tensors must be contiguous and fit the sizes")
         self._check(self.lib.lev_kv_write(_ptr(k), _ptr(v), _rows(k, "kv_write: k"), _rows(v, "kv_write: v"), _ptr(k_pages),
-                                          _ptr(v_pages), _ptr(dest), T, n_kv_heads, head_dim, page_size, _DT[dt], self._s()))
+                                          _ptr(v_pages), _ptr(dest), T, n_kv_heads, head_dim, vd, page_size, _DT[dt], self._s()))
+
+    # ---- row-wise steps of layers that are not GPT-2's -----------------------------------------
+    def head_prepare(self, qk, n_norm: int, head_dim: int, eps: float, v=None, v_first=None, n_blend: int = 0, value_dim: int = 0,
+                     blend=None) -> None:
+        """In place: the ``n_norm`` heads of ``head_dim`` columns at the start of ``qk``'s rows are divided by their root
+        mean square (``sqrt(mean(x^2) + eps)``); the ``n_blend`` heads of ``value_dim`` columns of ``v`` become
+        ``(1 - blend) v + blend v_first`` (``blend``: a float32 tensor of one element on the GPU). 32-bit arithmetic."""
+        T = (qk if qk is not None else v).shape[0]
+        dt = (qk if qk is not None else v).dtype
+        _dev(qk, v, v_first, blend)
+        _req(dt in _DT, "head_prepare: unknown dtype")
+        qs = vs = fs = 0
+        if n_norm:
+            _req(qk is not None and qk.shape[0] == T and qk.shape[1] >= n_norm * head_dim, "head_prepare: too few columns for the heads to normalise")
+            qs = _rows(qk, "head_prepare: qk")
+        if n_blend:
+            _req(v is not None and v_first is not None and blend is not None, "head_prepare: blending needs both value tensors and the weight")
+            _req(v.shape == v_first.shape == (T, n_blend * value_dim) and v.dtype == v_first.dtype == dt, "head_prepare: values must be [T, heads*value_dim]")
+            _req(blend.dtype == torch.float32 and blend.numel() == 1, "head_prepare: the blending weight must be one float32")
+            vs, fs = _rows(v, "head_prepare: v"), _rows(v_first, "head_prepare: v_first")
+        self._check(self.lib.lev_head_prepare(_ptr(qk) if n_norm else None, qs, int(n_norm), int(head_dim), float(eps), _ptr(v) if n_blend else None,
+                                              vs, _ptr(v_first) if n_blend else None, fs, int(n_blend), int(value_dim),
+                                              _ptr(blend) if n_blend else None, T, _DT[dt], self._s()))
+
+    def poly_norm(self, z, coefficients, eps: float, out) -> None:
+        """out = c0 z/rms(z) + c1 z^2/rms(z^2) + c2 z^3/rms(z^3) + c3 per row, rms(u) = sqrt(mean(u^2) + eps); powers element
+        by element, statistics in 32-bit. ``coefficients``: float32 [4] on the GPU."""
+        _dev(z, coefficients, out)
+        _req(z.dim() == 2 and out.shape == z.shape and z.dtype == out.dtype and z.dtype in _DT, "poly_norm: z and out must be [T, F] of one compute dtype")
+        _req(coefficients.dtype == torch.float32 and coefficients.numel() == 4 and coefficients.is_contiguous(), "poly_norm: four float32 coefficients")
+        self._check(self.lib.lev_poly_norm(_ptr(z), _rows(z, "poly_norm: z"), _ptr(out), _rows(out, "poly_norm: out"), _ptr(coefficients),
+                                           z.shape[0], z.shape[1], float(eps), _DT[z.dtype], self._s()))
+
+    def head_talk(self, o, talk, gate, out, n_heads: int, n_kv_heads: int, value_dim: int) -> None:
+        """``o`` float32 [T, heads, NV, value_dim] (``attention_values``) -> ``out`` [T, heads*value_dim] in the compute dtype:
+        head h gets ``sum_g talk[h, g] o[t, g, c(h)]`` with c(h) its own value head (``talk`` None: ``o[t, h, 0]``), times
+        ``sigmoid(gate[t, h])`` where ``gate`` [T, heads] (compute dtype) is given."""
+        _dev(o, talk, gate, out)
+        T = out.shape[0]
+        nv = n_kv_heads if talk is not None else 1
+        _req(o.dtype == torch.float32 and o.is_contiguous() and o.numel() == T * n_heads * nv * value_dim, "head_talk: o must be float32 [T, heads, NV, value_dim]")
+        _req(out.dtype in _DT and out.shape[1] == n_heads * value_dim, "head_talk: out must be [T, heads*value_dim]")
+        _req(talk is None or (talk.dtype == torch.float32 and talk.shape == (n_heads, n_heads) and talk.is_contiguous()), "head_talk: the mixing matrix must be float32 [heads, heads]")
+        gs = 0
+        if gate is not None:
+            _req(gate.dtype == out.dtype and gate.shape == (T, n_heads), "head_talk: the gate must be [T, heads] of the compute dtype")
+            gs = _rows(gate, "head_talk: gate")
+        self._check(self.lib.lev_head_talk(_ptr(o), _ptr(talk), _ptr(gate), gs, _ptr(out), _rows(out, "head_talk: out"), T, n_heads, n_kv_heads,
+                                           nv, value_dim, _DT[out.dtype], self._s()))
+
+    def stream_average(self, streams, x, weights, n: int) -> None:
+        """``streams`` float32 [slots, T, D] holds earlier results in entries 0 .. n-2. ``x`` (float32 [T, D]) is kept as entry
+        n-1 and becomes ``sum_j weights[j] streams[j]``, j = 0 .. n-1 in that order."""
+        _dev(streams, x, weights)
+        _req(x.dtype == streams.dtype == weights.dtype == torch.float32 and x.is_contiguous() and streams.is_contiguous(), "stream_average: contiguous float32 tensors")
+        _req(streams.dim() == 3 and streams.shape[1:] == x.shape and 1 <= n <= streams.shape[0], "stream_average: streams must be [slots >= n, T, D]")
+        _req(weights.numel() >= n and weights.is_contiguous(), "stream_average: one weight per stream")
+        self._check(self.lib.lev_stream_average(_ptr(streams), _ptr(x), _ptr(weights), int(n), x.numel(), self._s()))
+
+    def attention_values(self, q, out, k_pages, v_pages, meta, *, n_heads: int, n_kv_heads: int, head_dim: int, value_dim: int,
+                         all_value_heads: bool, page_size: int, scale: float, window: Optional[int], block_tables,
+                         softcap: Optional[float] = None, slopes=None) -> None:
+        """Causal attention over the pages for heads whose keys and values differ in size. ``out`` float32
+        [T, heads, NV, value_dim]: the weights of each query head applied to the values of every key/value head
+        (``all_value_heads``: NV = kv heads, for weights that are mixed over the heads afterwards, see ``head_talk``) or of its
+        own (NV = 1). Score: ``cap(scale q.k) - slopes[h] * distance`` (``slopes`` float32 [heads] or None), ``cap`` the soft
+        cap if given. The cache must hold the step's own keys and values already."""
+        _dev(q, out, k_pages, v_pages, block_tables, meta.positions, meta.token_seq, slopes)
+        T = q.shape[0]
+        dt = q.dtype
+        nv = n_kv_heads if all_value_heads else 1
+        _req(q.shape[1] == n_heads * head_dim and dt in _DT and dt == k_pages.dtype == v_pages.dtype, "attention_values: q must be [T, heads*head_dim] of the cache's dtype")
+        _req(out.dtype == torch.float32 and out.is_contiguous() and out.numel() == T * n_heads * nv * value_dim, "attention_values: out must be float32 [T, heads, NV, value_dim]")
+        _req(meta.positions.numel() == T and meta.token_seq.numel() == T, "attention_values: one position and request row per token")
+        _req(block_tables.dtype == torch.int32 and block_tables.dim() == 2 and block_tables.is_contiguous(), "attention_values: bad block tables")
+        _req(k_pages.is_contiguous() and v_pages.is_contiguous() and k_pages.numel() * value_dim == v_pages.numel() * head_dim
+             and k_pages.numel() % (n_kv_heads * head_dim * page_size) == 0, "attention_values: page tensors do not fit the sizes")
+        _req(slopes is None or (slopes.dtype == torch.float32 and slopes.numel() == n_heads and slopes.is_contiguous()), "attention_values: one float32 slope per head")
+        self._check(self.lib.lev_attention_values(
+            _ptr(q), _rows(q, "attention_values: q"), _ptr(out), _ptr(k_pages), _ptr(v_pages), _ptr(meta.positions), _ptr(meta.token_seq),
+            _ptr(block_tables), block_tables.shape[1], T, n_heads, n_kv_heads, head_dim, value_dim, nv, page_size, float(scale),
+            int(window) if window else 0, float(softcap) if softcap else 0.0, _ptr(slopes), _DT[dt], self._s()))
 
     # ---- attention -------------------------------------------------------------------------
     def paged_attention(self, q, out, k_pages, v_pages, meta, *, n_heads: int, n_kv_heads: int, head_dim: int,

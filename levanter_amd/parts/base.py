@@ -86,6 +86,9 @@ class StepContext:
     nobody: a mixer with state of its own must not count them). With ``attention.positions`` and
     ``attention.token_seq`` this is all a state mixer needs on the device, so that it can be ``graph_safe``."""
     units: Dict[int, CacheUnitView] = field(default_factory=dict)
+    shared: Dict[str, Any] = field(default_factory=dict)
+    """What parts of different layers hand each other within one step (the values of an earlier layer for the step's
+    tokens, the results of the layers so far). Empty when the step begins; nothing in it outlives the step."""
     pending: Any = None
     """A product into the residual stream that its kernel has not finished (``kernels.PendingSum``): the next norm of
     that tensor folds the rest in, anything else calls ``settle()`` first. Only set while ``may_defer`` is True."""
@@ -175,6 +178,18 @@ class FeedForward(Part):
     """``forward(h, x, ctx)``: adds the feed-forward's output for ``h`` to the residual ``x`` in place."""
 
     def forward(self, h: torch.Tensor, x: torch.Tensor, ctx: StepContext) -> None:
+        raise NotImplementedError
+
+
+class StreamMix(Part):
+    """Makes the residual stream that the next layer reads out of this layer's result and those of earlier layers.
+    ``enter(x, ctx)`` is called before the layer's parts read ``x`` (float32 ``[T, dim]``), ``leave(x, ctx)`` after they
+    have added to it: it replaces ``x`` in place. What it keeps of earlier layers lives in ``ctx.shared``."""
+
+    def enter(self, x: torch.Tensor, ctx: StepContext) -> None:
+        return None
+
+    def leave(self, x: torch.Tensor, ctx: StepContext) -> None:
         raise NotImplementedError
 
 

@@ -27,3 +27,33 @@ class PreNormBlock(Block):
         if not self.norm2.folds_pending:
             ctx.settle()
         self.feed_forward.forward(self.norm2(x, ctx), x, ctx)
+
+
+@BLOCKS.register("parallel")
+class ParallelBlock(Block):
+    """One norm whose output every branch reads: with h = norm1(x), x += mixer(h) + feed_forward(h). ``feed_forward`` may be
+    missing (a layer that only mixes). With a ``stream_mix`` part the sum is that layer's result, and what the next layer
+    reads is the mix's function of it and of earlier layers' results."""
+
+    roles = ("norm1", "mixer")
+
+    def __init__(self, parts: Dict[str, Part]):
+        super().__init__(parts)
+        unknown = [r for r in parts if r not in ("norm1", "mixer", "feed_forward", "stream_mix")]
+        if unknown:
+            raise ValueError(f"block 'parallel' has no role {', '.join(unknown)}")
+        self.norm1, self.mixer = parts["norm1"], parts["mixer"]
+        self.feed_forward = parts.get("feed_forward")
+        self.stream_mix = parts.get("stream_mix")
+
+    def forward(self, x: torch.Tensor, ctx: StepContext, unit: CacheUnitView, writes_cache: bool) -> None:
+        # both branches add to x and the mix reads it: the block does not say ``defers_residual``, so no product is ever
+        # left unfinished here
+        if self.stream_mix is not None:
+            self.stream_mix.enter(x, ctx)
+        h = self.norm1(x, ctx)
+        self.mixer.forward(h, x, ctx, unit, writes_cache)
+        if self.feed_forward is not None:
+            self.feed_forward.forward(h, x, ctx)
+        if self.stream_mix is not None:
+            self.stream_mix.leave(x, ctx)

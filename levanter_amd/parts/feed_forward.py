@@ -32,3 +32,31 @@ class DenseMlp(FeedForward):
     def forward(self, h: torch.Tensor, x: torch.Tensor, ctx: StepContext) -> None:
         m = self.up(h, ctx, activation=self.activation)
         self.down(m, ctx, residual=x, final=True)
+
+
+@FEED_FORWARDS.register("poly_norm_mlp")
+class PolyNormMlp(FeedForward):
+    """down(act(up(h))) with an activation that needs a token's whole row: c0 N(z) + c1 N(z^2) + c2 N(z^3) + c3, powers
+    element by element, N(u) = u / sqrt(mean(u^2) + eps) over the inner width. The statistics and the sum are 32-bit and
+    run as a kernel of their own between the two products. Tensors: ``up.weight``, ``down.weight`` (optional biases),
+    ``coefficients`` [4]."""
+
+    graph_safe = True
+
+    def __init__(self, spec: PartSpec, tensors: Dict[str, torch.Tensor], env: BuildEnv):
+        super().__init__(spec, tensors, env)
+        p = spec.params
+        layout = p.get("weight_layout", "out_in")
+        self.eps = float(p["eps"])
+        self.up = Linear(tensors["up.weight"], tensors.get("up.bias"), layout, env)
+        self.down = Linear(tensors["down.weight"], tensors.get("down.bias"), layout, env)
+        if (self.up.n_in, self.up.n_out) != (p["dim"], p["inner_dim"]) or (self.down.n_in, self.down.n_out) != (p["inner_dim"], p["dim"]):
+            raise ValueError("poly_norm_mlp: weights do not have the sizes of the description")
+        self.coefficients = tensors["coefficients"].to(env.device, torch.float32).contiguous()
+        if self.coefficients.numel() != 4:
+            raise ValueError(f"poly_norm_mlp: four coefficients, got {self.coefficients.numel()}")
+
+    def forward(self, h: torch.Tensor, x: torch.Tensor, ctx: StepContext) -> None:
+        z = self.up(h, ctx)
+        ctx.kernels.poly_norm(z, self.coefficients, self.eps, z)
+        self.down(z, ctx, residual=x, final=True)

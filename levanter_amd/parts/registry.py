@@ -1,5 +1,5 @@
 """Registries of part kinds. Each family (norm, position encoding, mixer, feed-forward, embedding,
-head, block) maps a kind name to a class; a model description names kinds, ``build_part`` constructs
+head, stream mix, block) maps a kind name to a class; a model description names kinds, ``build_part`` constructs
 them. Registering a new kind needs no change to the framework's files:
 
     @MIXERS.register("my_mixer")
@@ -48,9 +48,10 @@ FEED_FORWARDS: PartRegistry = PartRegistry("feed-forward")
 BLOCKS: PartRegistry = PartRegistry("block")
 HEADS: PartRegistry = PartRegistry("head")
 EMBEDDINGS: PartRegistry = PartRegistry("embedding")
+STREAM_MIXES: PartRegistry = PartRegistry("stream mix")
 
 FAMILIES: Dict[str, PartRegistry] = {"norm": NORMS, "position": POSITION_ENCODINGS, "mixer": MIXERS, "feed_forward": FEED_FORWARDS,
-                                     "embedding": EMBEDDINGS, "head": HEADS}
+                                     "embedding": EMBEDDINGS, "head": HEADS, "stream_mix": STREAM_MIXES}
 
 
 def part_class(kind: str, family: str = ""):

@@ -1,0 +1,136 @@
+"""Causal self-attention over the paged cache whose pieces are switched on by its description:
+
+* separate projections for queries, keys, values (and a gate), held as one matrix so that they are one product;
+* key and value heads of different sizes;
+* queries and keys divided by their root mean square per head (no weight);
+* a soft cap on the scaled score, then a term per head that grows with the distance, ``- slope[h] * (i - j)``;
+* a window of the last ``window`` keys;
+* the softmax weights mixed over the heads after the softmax, ``w'_h = sum_g talk[h, g] w_g``, each head applying its
+  mixed weights to the values of its own key/value head;
+* values blended with the values that an earlier layer computed for the same token (``value_mix``: the layer that is the
+  "source" leaves its values in ``ctx.shared``, a layer that says "blend" caches ``(1 - l) v + l v_source``);
+* the output of head h multiplied by ``sigmoid(gate_h(x))`` before the output projection.
+
+Scores, softmax, the unit norms, the blend and the mixing over heads are 32-bit in every precision. The mixing is done
+after the weights have been applied: the attention kernel gives, for every query head, its weights applied to the values
+of every key/value head, and a small kernel sums over the query heads (the two orders differ in rounding only).
+"""
+from __future__ import annotations
+
+from typing import Dict, Optional
+
+import torch
+
+from levanter_amd.cache.requirements import PagedKv
+from .base import BuildEnv, CacheUnitView, Mixer, StepContext
+from .linear import Linear
+from .registry import MIXERS
+from .spec import PartSpec
+
+
+def _pad8(n: int) -> int:
+    return (n + 7) // 8 * 8
+
+
+@MIXERS.register("talking_heads_attention")
+class TalkingHeadsAttention(Mixer):
+    """params: ``dim``, ``n_heads``, ``n_kv_heads``, ``head_dim``, ``value_dim``, ``scale``, ``window`` (None: all keys),
+    ``softcap`` (None: none), ``unit_norm_eps`` (None: queries and keys stay as projected), ``distance_slopes`` (one number
+    per head, or None), ``value_mix`` (None, "source" or "blend") and ``value_mix_key`` (the name under which layers that
+    belong together share values). Tensors: ``q.weight``, ``k.weight``, ``v.weight``, ``out.weight`` (``[out, in]``), their
+    optional ``.bias``, optional ``gate.weight`` ``[heads, dim]``, ``talk`` ``[heads, heads]``, ``value_mix.weight`` (one number)."""
+
+    graph_safe = True
+
+    def __init__(self, spec: PartSpec, tensors: Dict[str, torch.Tensor], env: BuildEnv):
+        super().__init__(spec, tensors, env)
+        p = spec.params
+        self.dim = int(p["dim"])
+        self.n_heads, self.n_kv_heads = int(p["n_heads"]), int(p["n_kv_heads"])
+        self.head_dim, self.value_dim = int(p["head_dim"]), int(p["value_dim"])
+        self.scale = float(p["scale"])
+        self.window: Optional[int] = p.get("window")
+        self.softcap = p.get("softcap")
+        self.unit_norm_eps = p.get("unit_norm_eps")
+        if self.n_heads % self.n_kv_heads != 0:
+            raise ValueError(f"attention: {self.n_heads} heads are not a multiple of {self.n_kv_heads} key/value heads")
+        if self.head_dim % 8 != 0 or self.value_dim % 8 != 0:
+            raise ValueError(f"attention: head sizes {self.head_dim} (keys) and {self.value_dim} (values) must be multiples of 8")
+        slopes = p.get("distance_slopes")
+        self.slopes = None
+        if slopes is not None:
+            if len(slopes) != self.n_heads:
+                raise ValueError(f"attention: {len(slopes)} slopes for {self.n_heads} heads")
+            self.slopes = torch.tensor([float(s) for s in slopes], dtype=torch.float32, device=env.device)
+        self.value_mix = p.get("value_mix")
+        if self.value_mix not in (None, "source", "blend"):
+            raise ValueError(f"attention: value_mix must be None, 'source' or 'blend', got {self.value_mix!r}")
+        self.value_mix_key = "value_mix." + str(p.get("value_mix_key", "values"))
+        self.blend = None
+        if self.value_mix == "blend":
+            self.blend = tensors["value_mix.weight"].to(env.device, torch.float32).reshape(1).contiguous()
+        talk = tensors.get("talk")
+        self.talk = None if talk is None else talk.to(env.device, torch.float32).contiguous()
+        if self.talk is not None and tuple(self.talk.shape) != (self.n_heads, self.n_heads):
+            raise ValueError(f"attention: the matrix that mixes the heads must be [{self.n_heads}, {self.n_heads}]")
+
+        # one matrix for all projections of the mixer's input: queries, keys, values, gate; each starts at a multiple of 8 columns
+        self.q_cols, self.k_cols, self.v_cols = self.n_heads * self.head_dim, self.n_kv_heads * self.head_dim, self.n_kv_heads * self.value_dim
+        names = ["q", "k", "v"] + (["gate"] if "gate.weight" in tensors else [])
+        sizes = {"q": self.q_cols, "k": self.k_cols, "v": self.v_cols, "gate": self.n_heads}
+        rows, biases, self.offsets, at = [], [], {}, 0
+        any_bias = any(f"{n}.bias" in tensors for n in names)
+        for n in names:
+            w = tensors[f"{n}.weight"].to(torch.float32)
+            if tuple(w.shape) != (sizes[n], self.dim):
+                raise ValueError(f"attention: {n}.weight must be [{sizes[n]}, {self.dim}], got {list(w.shape)}")
+            b = tensors.get(f"{n}.bias")
+            b = torch.zeros(sizes[n]) if b is None else b.to(torch.float32).cpu()
+            pad = _pad8(sizes[n]) - sizes[n]
+            self.offsets[n] = at
+            rows += [w.cpu(), torch.zeros(pad, self.dim)]
+            biases += [b, torch.zeros(pad)]
+            at += sizes[n] + pad
+        if self.offsets["k"] != self.q_cols:
+            raise ValueError("attention: heads * head_dim must be a multiple of 8 (keys follow the queries without a gap)")
+        self.proj = Linear(torch.cat(rows, 0), torch.cat(biases, 0) if any_bias else None, "out_in", env)
+        self.has_gate = "gate" in self.offsets
+        self.out = Linear(tensors["out.weight"], tensors.get("out.bias"), p.get("weight_layout", "out_in"), env)
+        if (self.out.n_in, self.out.n_out) != (self.n_heads * self.value_dim, self.dim):
+            raise ValueError("attention: the output projection does not have the sizes of the description")
+
+    def cache_requirement(self):
+        return PagedKv(self.n_kv_heads, self.head_dim, self.window, None if self.value_dim == self.head_dim else self.value_dim)
+
+    def forward(self, h: torch.Tensor, x: torch.Tensor, ctx: StepContext, unit: CacheUnitView, writes_cache: bool) -> None:
+        K = ctx.kernels
+        T = h.shape[0]
+        p = self.proj(h, ctx)  # [T, q | k | v | gate], compute dtype
+        o = self.offsets
+        q = p[:, :self.q_cols]
+        k = p[:, o["k"]:o["k"] + self.k_cols]
+        v = p[:, o["v"]:o["v"] + self.v_cols]
+        gate = p[:, o["gate"]:o["gate"] + self.n_heads] if self.has_gate else None
+        v_first = None
+        if self.value_mix == "source":
+            ctx.shared[self.value_mix_key] = v
+        elif self.value_mix == "blend":
+            v_first = ctx.shared.get(self.value_mix_key)
+            if v_first is None or v_first.shape != v.shape:
+                raise RuntimeError("attention: no layer before this one has left values of this shape to blend with")
+        n_norm = self.n_heads + self.n_kv_heads if self.unit_norm_eps is not None else 0
+        if n_norm or v_first is not None:
+            K.head_prepare(p[:, :self.q_cols + self.k_cols], n_norm, self.head_dim, self.unit_norm_eps or 0.0, v=v, v_first=v_first,
+                           n_blend=self.n_kv_heads if v_first is not None else 0, value_dim=self.value_dim, blend=self.blend)
+        g = unit.group
+        if writes_cache:
+            K.kv_write(k, v, unit.k_pages, unit.v_pages, g.dest, self.n_kv_heads, self.head_dim, g.page_size, value_dim=self.value_dim)
+        nv = self.n_kv_heads if self.talk is not None else 1
+        w = torch.empty((T, self.n_heads, nv, self.value_dim), dtype=torch.float32, device=h.device)
+        K.attention_values(q, w, unit.k_pages, unit.v_pages, ctx.attention, n_heads=self.n_heads, n_kv_heads=self.n_kv_heads,
+                           head_dim=self.head_dim, value_dim=self.value_dim, all_value_heads=self.talk is not None,
+                           page_size=g.page_size, scale=self.scale, window=self.window, block_tables=g.block_tables,
+                           softcap=self.softcap, slopes=self.slopes)
+        a = ctx.empty(T, self.n_heads * self.value_dim)
+        K.head_talk(w, self.talk, gate, a, self.n_heads, self.n_kv_heads, self.value_dim)
+        self.out(a, ctx, residual=x, final=True)

@@ -30,9 +30,18 @@ def random_tensors(spec: ModelSpec, seed: int, dtype: torch.dtype = torch.float3
         if ts.kind == "int":
             out[name] = torch.randint(0, 1 << 15, ts.shape, generator=g, device=dev, dtype=torch.int32)
             continue
-        t = torch.empty(ts.shape, device=dev, dtype=torch.float32).normal_(0.0, spec.init_std, generator=g)
+        std = spec.init_std if ts.std is None else float(ts.std)
+        t = torch.empty(ts.shape, device=dev, dtype=torch.float32).normal_(0.0, std, generator=g)
         if ts.init == "one_plus_normal":
             t += 1.0
+        elif ts.init == "eye_plus_normal":
+            t += torch.eye(ts.shape[0], ts.shape[1], device=dev)
+        elif ts.init == "last_one_plus_normal":
+            t.view(-1)[-1] += 1.0
+        elif ts.init == "unit_interval":
+            t = torch.empty(ts.shape, device=dev, dtype=torch.float32).uniform_(0.1, 0.9, generator=g)
+        elif ts.init != "normal":
+            raise ValueError(f"tensor {name}: unknown way to draw it, {ts.init!r}")
         out[name] = t.to(dtype)
     return out
 

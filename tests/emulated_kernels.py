@@ -111,21 +111,22 @@ class EmulatedKernels:
     def v_view(v_pages, kvh, hd, ps):
         return v_pages.view(-1, kvh, hd, ps)
 
-    def kv_write(self, k, v, k_pages, v_pages, dest, n_kv_heads, head_dim, page_size) -> None:
+    def kv_write(self, k, v, k_pages, v_pages, dest, n_kv_heads, head_dim, page_size, value_dim=None) -> None:
+        vd = head_dim if value_dim is None else value_dim
         kv_ = self.k_view(k_pages, n_kv_heads, head_dim, page_size)
-        vv_ = self.v_view(v_pages, n_kv_heads, head_dim, page_size)
+        vv_ = self.v_view(v_pages, n_kv_heads, vd, page_size)
         for t in range(k.shape[0]):
             d = int(dest[t])
             if d < 0:
                 continue
             page, off = d // page_size, d % page_size
             kv_[page, :, :, off, :] = k[t].view(n_kv_heads, head_dim // 8, 8)
-            vv_[page, :, :, off] = v[t].view(n_kv_heads, head_dim)
+            vv_[page, :, :, off] = v[t].view(n_kv_heads, vd)
 
-    def gather_kv(self, k_pages, v_pages, table_row, lo, hi, n_kv_heads, head_dim, page_size):
-        """Keys and values of positions lo..hi-1 of one request: [kvh, n, hd] each."""
+    def gather_kv(self, k_pages, v_pages, table_row, lo, hi, n_kv_heads, head_dim, page_size, value_dim=None):
+        """Keys and values of positions lo..hi-1 of one request: [kvh, n, hd] (values [kvh, n, value_dim])."""
         kv_ = self.k_view(k_pages, n_kv_heads, head_dim, page_size)
-        vv_ = self.v_view(v_pages, n_kv_heads, head_dim, page_size)
+        vv_ = self.v_view(v_pages, n_kv_heads, head_dim if value_dim is None else value_dim, page_size)
         ks, vs = [], []
         for p in range(lo, hi):
             page = int(table_row[p // page_size])
@@ -161,6 +162,65 @@ class EmulatedKernels:
             o = torch.einsum("hn,hnd->hd", p, vs)
             out[t] = o.reshape(-1).to(out.dtype)
         return False
+
+    # ---- row-wise steps of layers that are not GPT-2's
+    def head_prepare(self, qk, n_norm, head_dim, eps, v=None, v_first=None, n_blend=0, value_dim=0, blend=None) -> None:
+        if n_norm:
+            x = qk[:, :n_norm * head_dim].float().view(qk.shape[0], n_norm, head_dim)
+            x = x / torch.sqrt((x * x).mean(-1, keepdim=True) + eps)
+            qk[:, :n_norm * head_dim] = x.reshape(qk.shape[0], -1).to(qk.dtype)
+        if n_blend:
+            lam = float(blend.reshape(-1)[0])
+            v.copy_(((1.0 - lam) * v.float() + lam * v_first.float()).to(v.dtype))
+
+    def poly_norm(self, z, coefficients, eps, out) -> None:
+        u = z.float()
+        c = [float(x) for x in coefficients]
+
+        def n(w):
+            return w / torch.sqrt((w * w).mean(-1, keepdim=True) + eps)
+
+        out.copy_((c[0] * n(u) + c[1] * n(u * u) + c[2] * n(u * u * u) + c[3]).to(out.dtype))
+
+    def head_talk(self, o, talk, gate, out, n_heads, n_kv_heads, value_dim) -> None:
+        T = out.shape[0]
+        if talk is None:
+            a = o.view(T, n_heads, value_dim)
+        else:
+            ov = o.view(T, n_heads, n_kv_heads, value_dim)
+            own = torch.arange(n_heads) // (n_heads // n_kv_heads)
+            a = torch.einsum("hg,tghd->thd", talk.float(), ov[:, :, own, :])  # [t, g, h, d]: weights of g on the values of h's own head
+        if gate is not None:
+            a = a * torch.sigmoid(gate.float())[:, :, None]
+        out.copy_(a.reshape(T, -1).to(out.dtype))
+
+    def stream_average(self, streams, x, weights, n) -> None:
+        streams[n - 1].copy_(x)
+        acc = torch.zeros_like(x)
+        for j in range(n):
+            acc += weights[j] * streams[j]
+        x.copy_(acc)
+
+    def attention_values(self, q, out, k_pages, v_pages, meta, *, n_heads, n_kv_heads, head_dim, value_dim, all_value_heads, page_size,
+                         scale, window, block_tables, softcap=None, slopes=None) -> None:
+        T = q.shape[0]
+        g = n_heads // n_kv_heads
+        o = out.view(T, n_heads, n_kv_heads if all_value_heads else 1, value_dim)
+        for t in range(T):
+            pos = int(meta.positions[t])
+            row = block_tables[int(meta.token_seq[t])]
+            lo = max(0, pos - window + 1) if window else 0
+            ks, vs = self.gather_kv(k_pages, v_pages, row, lo, pos + 1, n_kv_heads, head_dim, page_size, value_dim)
+            s = torch.einsum("hd,hnd->hn", q[t].float().view(n_heads, head_dim), ks.float().repeat_interleave(g, 0)) * scale
+            if softcap:
+                s = softcap * torch.tanh(s / softcap)
+            if slopes is not None:
+                s = s - slopes.float()[:, None] * (pos - torch.arange(lo, pos + 1)).float()[None, :]
+            p = torch.softmax(s, -1)
+            if all_value_heads:
+                o[t] = torch.einsum("hn,cnd->hcd", p, vs.float())
+            else:
+                o[t, :, 0] = torch.einsum("hn,hnd->hd", p, vs.float().repeat_interleave(g, 0))
 
     # ---- sampling
     def sample(self, logits, temperatures, keys, positions, out_tokens, out_logprobs) -> None:
