@@ -55,9 +55,12 @@ def main() -> int:
     ap.add_argument("--shape", default="7b", choices=["7b", "xl", "20b"],
                     help="layer sizes of the decode workload: 7b is the headline's; xl and 20b measure the same step at the other "
                          "sizes of the reference's configurations (use --no-points: the prefill point is 2,048 tokens)")
-    ap.add_argument("--workload", default="decode", choices=["decode", "xl_mix", "20b"],
+    ap.add_argument("--workload", default="decode", choices=["decode", "xl_mix", "20b", "zederax"],
                     help="decode: the workload described above. xl_mix / 20b: continuous-batching workloads at the gpt2_xl and gpt2_20b sizes "
-                         "through InferenceEngine.generate; they print their own line")
+                         "through InferenceEngine.generate; they print their own line. zederax: prefill and decode rates of Zederax "
+                         "layers at a few sizes beside GPT-2 layers of the same width, heads and inner width; its own line")
+    ap.add_argument("--sizes", default="1k,2k,4k", help="with --workload zederax: which of the sizes 1k, 2k, 4k to run")
+    ap.add_argument("--arch", default="both", choices=["both", "zederax", "gpt2"], help="with --workload zederax: one architecture only (for profiling)")
     args = ap.parse_args()
     if args.gpus != 1:
         print(f"bench.py: this engine runs on one GPU; --gpus {args.gpus} is not supported")
@@ -68,6 +71,8 @@ def main() -> int:
     from levanter_amd.config import InferenceEngineConfig, LmConfig
     from levanter_amd.engine import InferenceEngine, Request
 
+    if args.workload == "zederax":
+        return zederax_workload(args)
     if args.workload != "decode":
         return serving_workload(args)
 
@@ -289,6 +294,105 @@ def serving_workload(args) -> int:
         "preemptions": engine.scheduler.n_preemptions,
     }
     print(json.dumps(out), flush=True)
+    return 0
+
+
+# Zederax layers at sizes that resemble real models' (width, query heads, key/value heads, key and value head size, inner
+# width, layers, window), and GPT-2 layers of the same width, heads and inner width beside them
+ZEDERAX_SIZES = {
+    "1k": dict(width=1024, heads=16, kv_heads=4, dim=64, vdim=64, ff=4096, layers=8, window=1024),
+    "2k": dict(width=2048, heads=16, kv_heads=4, dim=128, vdim=64, ff=8192, layers=8, window=1024),
+    "4k": dict(width=4096, heads=32, kv_heads=8, dim=128, vdim=128, ff=16384, layers=4, window=2048),
+}
+ZEDERAX_VOCAB = 32000
+
+
+def zederax_config(z):
+    import math
+
+    mixer = {"heads": z["heads"], "kv_heads": z["kv_heads"], "dim": z["dim"], "vdim": z["vdim"], "scale": 1.0 / math.sqrt(z["dim"]) * 4.0,
+             "softcap": 30.0, "mask": {"size": z["window"]}, "v_mix": True}
+    return {"architecture": "Zederax", "vocab": ZEDERAX_VOCAB, "width": z["width"], "norm": {"eps": 1e-6},
+            "layers": [{"type": "attention", "mixer": dict(mixer), "mlp": {"kind": "dense", "ff": z["ff"]}} for _ in range(z["layers"])]}
+
+
+def gpt2_config_like(z):
+    return {"model_type": "gpt2", "n_layer": z["layers"], "n_embd": z["width"], "n_head": z["heads"], "n_inner": z["ff"],
+            "vocab_size": ZEDERAX_VOCAB, "n_positions": 4096, "layer_norm_epsilon": 1e-5, "activation_function": "gelu_new"}
+
+
+def zederax_workload(args) -> int:
+    """Prefill (one 2,048-token prompt) and decode (batch 1, 8, 64 after 512-token prompts) through the engine, for Zederax
+    and for GPT-2 at equal sizes. One JSON line."""
+    import torch
+
+    from levanter_amd.config import InferenceEngineConfig, LmConfig
+    from levanter_amd.engine import InferenceEngine, Request
+
+    ps, prompt_len, V = 16, 512, ZEDERAX_VOCAB
+    steps, warmup = min(args.steps, 128), args.warmup
+    batches = (1, 8, 64)
+    ctx_end = prompt_len + 64 + warmup + steps + 16
+    pages_per_seq = (max(ctx_end, 2048) + ps - 1) // ps
+
+    def prompts(batch, n, seed):
+        g = torch.Generator().manual_seed(seed)
+        return [torch.randint(0, V, (n,), generator=g).tolist() for _ in range(batch)]
+
+    def measure(raw):
+        ecfg = InferenceEngineConfig(max_pages=max(batches) * ((ctx_end + ps - 1) // ps) + pages_per_seq, max_seqs=max(batches), page_size=ps,
+                                     max_pages_per_seq=pages_per_seq, compute_dtype=args.dtype, max_prefill_size=2048,
+                                     max_seqs_in_prefill=max(batches))
+        engine = InferenceEngine.from_config(LmConfig.from_dict(raw), seed=0, config=ecfg)
+        out = {"weights_gb": round(engine.model.weight_bytes() / 1e9, 3)}
+        times = []
+        for rep in range(4):
+            engine.reset()
+            engine.enqueue_requests([Request(prompt_tokens=prompts(1, 2048, 50 + rep)[0], request_id=rep, max_new_tokens=1)])
+            torch.cuda.synchronize()
+            t = time.perf_counter()
+            engine.step()
+            torch.cuda.synchronize()
+            if rep > 0:
+                times.append(time.perf_counter() - t)
+        out["prefill_2048_tok_s"] = round(2048 / sorted(times)[len(times) // 2], 1)
+        for b in batches:
+            engine.reset()
+            reqs = [Request(prompt_tokens=p, request_id=i, max_new_tokens=64 + warmup + steps + 8, temperature=0.0)
+                    for i, p in enumerate(prompts(b, prompt_len, b))]
+            seqs = engine.enqueue_requests(reqs)
+            while any(s.n_cached < s.prompt_len for s in seqs) or any(not s.generated for s in seqs):
+                engine.step()
+            for _ in range(warmup):
+                engine.step()
+            torch.cuda.synchronize()
+            t = time.perf_counter()
+            for _ in range(steps):
+                engine.step()
+            torch.cuda.synchronize()
+            dt = time.perf_counter() - t
+            assert all(not s.done for s in seqs)
+            out[f"decode_b{b}_tok_s"] = round(b * steps / dt, 1)
+            out[f"decode_b{b}_ms_per_step"] = round(dt / steps * 1e3, 4)
+        engine.reset()
+        del engine
+        torch.cuda.empty_cache()
+        return out
+
+    results = {}
+    for name in args.sizes.split(","):
+        if name not in ZEDERAX_SIZES:
+            print(f"bench.py: unknown size {name!r}; known: {', '.join(ZEDERAX_SIZES)}")
+            return 2
+        z = ZEDERAX_SIZES[name]
+        results[name] = {"sizes": z}
+        for arch, raw in (("zederax", zederax_config(z)), ("gpt2", gpt2_config_like(z))):
+            if args.arch in ("both", arch):
+                print(f"[bench] {arch} at size {name} ...", file=sys.stderr, flush=True)
+                results[name][arch] = measure(raw)
+    print(json.dumps({"metric": "prefill and decode tok/s of Zederax layers beside GPT-2 layers of equal width, heads and inner width",
+                      "unit": "tok/s", "n_gpus": 1, "steps": steps, "warmup": warmup, "dtype": "bf16" if args.dtype == "bfloat16" else "fp32",
+                      "data": "synthetic (random weights, uniform-random token ids)", "results": results}), flush=True)
     return 0
 
 

@@ -1,0 +1,246 @@
+// The attention of attention_values.hip on the matrix cores, bfloat16 in, 32-bit softmax and accumulation. Compiled once
+// per pair of head sizes: -DLEV_HD=<key head size> -DLEV_VD=<value head size>, both multiples of 16.
+//
+// As in attention_mfma.hip the problem is transposed so that no operand needs a transposition:
+//   S^T = K . Q^T      A operand: 16 keys x 32 head dims from the key pages, B operand: Q^T, in registers
+//   O^T = V^T . P^T    A operand: 16 value dims x 32 keys from the transposed value pages, B operand: P^T, which is what
+//                      the lanes hold after the softmax
+// with the 16x16x32 MFMA (A lane l: row l%16, k = 8*(l/16) .. +7; B lane l: column l%16, the same k; accumulator register
+// r of lane l: row 4*(l/16) + r, column l%16). The rows of score tile (u, h) are the keys 32u + 8*(row/4) + 4h + row%4 of
+// a block of 64, so that lane group g = l/16 holds the weights of the keys 32u + 8g .. +7 in its two tiles.
+//
+// One wave owns 16 columns that share a request and a key/value head:
+//   * a run of several tokens: 16 consecutive query tokens of one query head;
+//   * a single token: the query heads of one key/value head (up to 16 at a time).
+// It walks the keys in blocks of 64 (operands go from the pages straight into registers), keeps a running maximum and sum
+// per column, and applies the weights to the values of `nvc` value heads (blockIdx.z picks which): its own one, or, for
+// layers that mix the weights over the heads afterwards, every key/value head in turn.
+//
+//   score(t, key) = cap(scale * q . k) - slope[h] * (position(t) - position(key)),  cap(s) = softcap * tanh(s / softcap)
+//   out [T][H][NV][VD] float32, as attention_values.hip writes it.
+#include "common.h"
+#include "attention_config.h"
+
+#if !defined(LEV_HD) || !defined(LEV_VD)
+#error "compile with -DLEV_HD=<key head size> -DLEV_VD=<value head size>"
+#endif
+
+typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
+typedef __attribute__((ext_vector_type(4))) float f32x4;
+typedef __attribute__((ext_vector_type(4))) uint32_t u32x4;
+
+#define HD LEV_HD
+#define VD LEV_VD
+#define NKS ((HD + 31) / 32)  // k-steps of the score product
+#define NDT (VD / 16)         // 16-row tiles of O^T per value head
+// value heads per wave: at most 16 accumulator tiles (64 registers)
+#define NVC (NDT <= 2 ? 8 : (NDT <= 4 ? 4 : (NDT <= 8 ? 2 : 1)))
+#define SUB_TILES (PF_ROWS / 16)
+
+__device__ __forceinline__ bf16x8 as_bf16x8(u32x4 v) {
+  union { u32x4 u; bf16x8 b; } c;
+  c.u = v;
+  return c.b;
+}
+
+// all but the first n of eight consecutive keys' values (two to a word) made zero: what lies behind the last key that was
+// written may be anything, NaN too, and zero times that would reach the sum
+__device__ __forceinline__ u32x4 first_keys(u32x4 v, int n) {
+#pragma unroll
+  for (int e = 0; e < 4; ++e) v[e] &= n >= 2 * e + 2 ? 0xffffffffu : (n == 2 * e + 1 ? 0x0000ffffu : 0u);
+  return v;
+}
+
+__device__ __forceinline__ float fast_tanh(float x) {  // 1 - 2 / (1 + e^(2x)) with the hardware's exp2 and reciprocal
+  return 1.0f - 2.0f * __builtin_amdgcn_rcpf(1.0f + __builtin_amdgcn_exp2f(x * 2.8853900817779268f));
+}
+
+template <bool SINGLE>
+__global__ void __launch_bounds__(64)
+attention_values_mfma_kernel(const bf16_t* __restrict__ q, long q_stride, float* __restrict__ out, const bf16_t* __restrict__ k_pages,
+                             const bf16_t* __restrict__ v_pages, const int* __restrict__ positions, const int* __restrict__ token_seq,
+                             const int* __restrict__ block_tables, int bt_stride, const int* __restrict__ work, int H, int KVH, int NV,
+                             int PS, float scale, int window, float softcap, const float* __restrict__ slopes) {
+  const int lane = threadIdx.x, col = lane & 15, g = lane >> 4;
+  const int group = H / KVH;
+  int tok = 0, head = 0, kvh = 0;
+  bool valid;
+  if (SINGLE) {
+    const int col_sets = (group + 15) / 16;
+    kvh = blockIdx.y / col_sets;
+    const int c = (blockIdx.y % col_sets) * 16 + col;
+    valid = c < group;
+    head = kvh * group + (valid ? c : 0);
+    tok = work[blockIdx.x];
+  } else {
+    const int tile = blockIdx.x / SUB_TILES, sub = blockIdx.x % SUB_TILES;
+    const int first = work[2 * tile], n = work[2 * tile + 1];
+    if (sub * 16 >= n) return;  // the whole wave
+    head = blockIdx.y;
+    kvh = head / group;
+    valid = sub * 16 + col < n;
+    tok = first + (valid ? sub * 16 + col : sub * 16);
+  }
+  const int pos = positions[tok];
+  const int lo = window > 0 ? max(0, pos - window + 1) : 0;
+  // the wave's range of keys; every column belongs to the same request
+  int p_max = valid ? pos : -1, lo_min = valid ? lo : 0x7fffffff;
+#pragma unroll
+  for (int o = 8; o > 0; o >>= 1) {
+    p_max = max(p_max, __shfl_xor(p_max, o, 64));
+    lo_min = min(lo_min, __shfl_xor(lo_min, o, 64));
+  }
+  const int* bt = block_tables + (size_t)token_seq[tok] * bt_stride;
+  const float slope = slopes ? slopes[head] : 0.f;
+  const int c0 = NV == 1 ? kvh : blockIdx.z * NVC;             // first value head of this wave
+  const int n_c = NV == 1 ? 1 : min(NVC, NV - blockIdx.z * NVC);  // and how many
+
+  u32x4 qf[NKS];
+#pragma unroll
+  for (int s = 0; s < NKS; ++s) {
+    qf[s] = u32x4{0u, 0u, 0u, 0u};
+    if (valid && 32 * s + 8 * g < HD)
+      qf[s] = *reinterpret_cast<const u32x4*>(q + (size_t)tok * q_stride + (size_t)head * HD + 32 * s + 8 * g);
+  }
+  f32x4 o[NVC][NDT];
+#pragma unroll
+  for (int c = 0; c < NVC; ++c)
+#pragma unroll
+    for (int dt = 0; dt < NDT; ++dt) o[c][dt] = f32x4{0.f, 0.f, 0.f, 0.f};
+  float m = -INFINITY, l = 0.f;
+  constexpr float LOG2E = 1.4426950408889634f;
+  const size_t k_head = (size_t)HD * PS, v_head = (size_t)VD * PS;
+
+  for (int key0 = (lo_min / 64) * 64; key0 <= p_max; key0 += 64) {
+    // pages of this lane's two groups of 8 keys (32u + 8g .. +7): for the mask and for the values
+    int pgv[2];
+#pragma unroll
+    for (int u = 0; u < 2; ++u) {
+      const int kp = key0 + 32 * u + 8 * g;
+      pgv[u] = kp <= p_max ? bt[kp / PS] : -1;
+    }
+    // scores: S^T tiles (u, h)
+    f32x4 st[2][2];
+#pragma unroll
+    for (int u = 0; u < 2; ++u)
+#pragma unroll
+      for (int hh = 0; hh < 2; ++hh) {
+        const int kp = key0 + 32 * u + 8 * (col >> 2) + 4 * hh + (col & 3);  // the key of this lane's operand row
+        int page = kp <= p_max ? bt[kp / PS] : -1;
+        page = max(page, 0);  // a key without a page is masked below; its operand may be anything that can be read
+        const bf16_t* kb = k_pages + ((size_t)page * KVH + kvh) * k_head + (size_t)(kp % PS) * 8;
+        f32x4 acc = f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int s = 0; s < NKS; ++s) {
+          u32x4 kf = u32x4{0u, 0u, 0u, 0u};
+          if (32 * s + 8 * g < HD) kf = *reinterpret_cast<const u32x4*>(kb + (size_t)(4 * s + g) * PS * 8);
+          acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_bf16x8(kf), as_bf16x8(qf[s]), acc, 0, 0, 0);
+        }
+        st[u][hh] = acc;
+      }
+    // scale, cap, distance term, mask; in base 2 from here on
+    float mx = -INFINITY;
+#pragma unroll
+    for (int u = 0; u < 2; ++u)
+#pragma unroll
+      for (int hh = 0; hh < 2; ++hh)
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+          const int kp = key0 + 32 * u + 8 * g + 4 * hh + r;
+          const bool ok = valid && kp <= pos && kp >= lo && pgv[u] >= 0;
+          float s = st[u][hh][r] * scale;
+          if (softcap > 0.f) s = softcap * fast_tanh(s * __builtin_amdgcn_rcpf(softcap));
+          s = (s - slope * (float)(pos - kp)) * LOG2E;
+          s = ok ? s : -INFINITY;
+          st[u][hh][r] = s;
+          mx = fmaxf(mx, s);
+        }
+    mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
+    mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
+    const float m_new = fmaxf(m, mx);
+    const float m_use = m_new == -INFINITY ? 0.f : m_new;
+    const float corr = __builtin_amdgcn_exp2f(m - m_use);  // m = -inf: 0
+    m = m_new;
+    float psum = 0.f;
+    u32x4 pf[2];
+#pragma unroll
+    for (int u = 0; u < 2; ++u) {
+      float p[8];
+#pragma unroll
+      for (int hh = 0; hh < 2; ++hh)
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+          p[4 * hh + r] = __builtin_amdgcn_exp2f(st[u][hh][r] - m_use);
+          psum += p[4 * hh + r];
+        }
+#pragma unroll
+      for (int e = 0; e < 4; ++e) pf[u][e] = float2_to_bf16x2(p[2 * e], p[2 * e + 1]);
+    }
+    l = l * corr + psum;
+    // values of every value head of this wave
+#pragma unroll
+    for (int c = 0; c < NVC; ++c) {
+      if (c < n_c) {
+#pragma unroll
+        for (int dt = 0; dt < NDT; ++dt) {
+          f32x4 acc = o[c][dt] * corr;
+#pragma unroll
+          for (int u = 0; u < 2; ++u) {
+            const int kp = key0 + 32 * u + 8 * g;
+            const bf16_t* vb = v_pages + ((size_t)max(pgv[u], 0) * KVH + (c0 + c)) * v_head + (size_t)(16 * dt + col) * PS + kp % PS;
+            u32x4 vf = *reinterpret_cast<const u32x4*>(vb);
+            vf = first_keys(vf, pgv[u] >= 0 ? min(8, max(0, p_max - kp + 1)) : 0);
+            acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_bf16x8(vf), as_bf16x8(pf[u]), acc, 0, 0, 0);
+          }
+          o[c][dt] = acc;
+        }
+      }
+    }
+  }
+  l += __shfl_xor(l, 16, 64);
+  l += __shfl_xor(l, 32, 64);
+  if (!valid) return;
+  const float inv = l > 0.f ? 1.0f / l : 0.f;
+#pragma unroll
+  for (int c = 0; c < NVC; ++c) {
+    if (c < n_c) {
+      float* ob = out + (((size_t)tok * H + head) * NV + (NV == 1 ? 0 : c0 + c)) * VD;
+#pragma unroll
+      for (int dt = 0; dt < NDT; ++dt) *reinterpret_cast<f32x4*>(ob + 16 * dt + 4 * g) = o[c][dt] * inv;
+    }
+  }
+}
+
+extern "C" int lev_attention_values_mfma(const void* q, long q_stride, float* out, const void* k_pages, const void* v_pages,
+                                         const int* positions, const int* token_seq, const int* block_tables, int bt_stride,
+                                         const int* tiles, int n_tiles, const int* singles, int n_singles, int H, int KVH, int HD_,
+                                         int VD_, int NV, int PS, float scale, int window, float softcap, const float* slopes,
+                                         hipStream_t stream) {
+  LEV_REQUIRE(HD_ == HD && VD_ == VD, "attention: this library was built for head sizes %d / %d, not %d / %d", HD, VD, HD_, VD_);
+  LEV_REQUIRE(H > 0 && KVH > 0 && H % KVH == 0, "attention: bad head counts heads=%d kv_heads=%d", H, KVH);
+  LEV_REQUIRE(NV == 1 || NV == KVH, "attention: %d value heads per query head (1 or kv_heads=%d)", NV, KVH);
+  LEV_REQUIRE(PS > 0 && PS % 16 == 0, "attention: page_size=%d must be a multiple of 16", PS);
+  LEV_REQUIRE(window >= 0 && softcap >= 0.f, "attention: window=%d and soft cap %g must not be negative", window, (double)softcap);
+  LEV_REQUIRE(n_tiles >= 0 && n_singles >= 0 && (n_tiles == 0 || tiles) && (n_singles == 0 || singles), "attention: bad work lists");
+  LEV_REQUIRE(((uintptr_t)q & 15) == 0 && q_stride % 8 == 0 && ((uintptr_t)k_pages & 15) == 0 && ((uintptr_t)v_pages & 15) == 0 &&
+                  ((uintptr_t)out & 15) == 0,
+              "attention: operands must be 16-byte aligned");
+  const int chunks = NV == 1 ? 1 : (NV + NVC - 1) / NVC;
+  LEV_REQUIRE(H <= 65535 && chunks <= 65535, "attention: too many heads (%d)", H);
+  if (n_tiles > 0) {
+    dim3 grid(n_tiles * SUB_TILES, H, chunks);
+    attention_values_mfma_kernel<false><<<grid, 64, 0, stream>>>((const bf16_t*)q, q_stride, out, (const bf16_t*)k_pages,
+                                                                (const bf16_t*)v_pages, positions, token_seq, block_tables, bt_stride,
+                                                                tiles, H, KVH, NV, PS, scale, window, softcap, slopes);
+    if (lev_check_launch("attention_values_mfma (runs)")) return -1;
+  }
+  if (n_singles > 0) {
+    const int group = H / KVH;
+    dim3 grid(n_singles, KVH * ((group + 15) / 16), chunks);
+    attention_values_mfma_kernel<true><<<grid, 64, 0, stream>>>((const bf16_t*)q, q_stride, out, (const bf16_t*)k_pages,
+                                                               (const bf16_t*)v_pages, positions, token_seq, block_tables, bt_stride,
+                                                               singles, H, KVH, NV, PS, scale, window, softcap, slopes);
+    if (lev_check_launch("attention_values_mfma (single tokens)")) return -1;
+  }
+  return 0;
+}

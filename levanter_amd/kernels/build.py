@@ -4,7 +4,9 @@
   the 32-bit attentions;
 * ``gemm_mfma``: the bfloat16 GEMMs on the matrix cores;
 * ``gemm_library``: the vendor library's GEMM (hipBLASLt) for prompt-sized row counts, where it is ahead;
-* ``attn_hd<N>``: the bfloat16 attention on the matrix cores for head size N (16 .. 128 in steps of 16).
+* ``attn_hd<N>``: the bfloat16 attention on the matrix cores for head size N (16 .. 128 in steps of 16);
+* ``attnv_hd<N>_vd<M>``: the bfloat16 attention for key heads of N and value heads of M whose weights may be applied to
+  every value head (layers that mix their weights over the heads); a few pairs are registered here, others at first use.
 
 A model loads ``core`` and, in bfloat16, ``gemm_mfma`` and the attention unit of its own head size, so a first
 call in a fresh checkout compiles what that model needs. The libraries are built in the tree
@@ -80,6 +82,18 @@ def unregister_unit(name: str) -> None:
 
 def attention_unit(head_dim: int) -> str:
     return f"attn_hd{head_dim}"
+
+
+def attention_values_unit(head_dim: int, value_dim: int) -> str:
+    """The unit of the matrix-core attention for key heads of ``head_dim`` and value heads of ``value_dim`` (multiples of
+    16, at most 256); a pair that is not among the pre-registered ones is registered here, and compiled at its first use."""
+    name = f"attnv_hd{head_dim}_vd{value_dim}"
+    if name not in UNITS:
+        if head_dim % 16 or value_dim % 16 or not (16 <= head_dim <= 256 and 16 <= value_dim <= 256):
+            raise ValueError(f"no matrix-core attention for head sizes {head_dim} / {value_dim}")
+        register_unit(name, [("attention_values_mfma.hip", [f"-DLEV_HD={head_dim}", f"-DLEV_VD={value_dim}"], f"attention_values_mfma_hd{head_dim}_vd{value_dim}.o")],
+                      signatures={"lev_attention_values_mfma": [_P, _L, _P, _P, _P, _P, _P, _P, _I, _P, _I, _P, _I] + [_I] * 6 + [_F, _I, _F, _P, _P]})
+    return name
 
 
 def lib_name(unit: str) -> str:
@@ -290,3 +304,6 @@ for _hd in MFMA_ATTENTION_HEAD_DIMS:
                                         ("attention_dispatch.hip", [f"-DLEV_HD={_hd}"], f"attention_dispatch_hd{_hd}.o")], signatures={
         "lev_attention_mfma": [_P, _L, _P, _L, _P, _P, _P, _P, _P, _I, _P, _I, _P, _I, _P, _P, _L, _P, _P] + [_I] * 5 + [_F, _I, _F, _P, _I, _P],
     })
+# key / value head sizes of the attention with separate sizes that are built ahead; any other pair is built at its first use
+for _hd, _vd in ((32, 16), (16, 32), (48, 32), (64, 64), (128, 64), (128, 128)):
+    attention_values_unit(_hd, _vd)
