@@ -450,6 +450,82 @@ class HipKernels:
     def mfma_attention_values_supports(head_dim: int, value_dim: int) -> bool:
         return head_dim % 16 == 0 and value_dim % 16 == 0 and 16 <= head_dim <= 256 and 16 <= value_dim <= 256
 
+    # ---- attention -------------------------------------------------------------------------
+    def paged_attention(self, q, out, k_pages, v_pages, meta, *, n_heads: int, n_kv_heads: int, head_dim: int,
+                        page_size: int, scale: float, window: Optional[int], block_tables, k_new=None, v_new=None,
+                        dest=None, softcap: Optional[float] = None, score_bias=None) -> bool:
+        """Causal attention of the step's query tokens over the pages. ``meta`` is the step's
+        ``AttentionMeta`` (positions, token_seq and the work lists), block_tables int32 [S, B].
+
+        ``score_bias`` (float32 ``[n_heads, L]``): entry ``[h, min(d, L - 1)]`` is added to the scaled score of head ``h``
+        for a key ``d`` positions behind its query; ``softcap``: scores become ``softcap * tanh(score / softcap)`` (after
+        the bias, before the mask). Both off by default.
+
+        ``k_new``/``v_new``/``dest``: the step's new keys and values, not yet written. Returns True if this
+        call has written them to their pages (a step of single tokens on the matrix-core path does it inside
+        the attention kernel); False means the caller must call ``kv_write`` first and call again without them."""
+        if not (q.is_cuda and out.is_cuda and k_pages.is_cuda and v_pages.is_cuda):
+            raise KernelError("a kernel was given a tensor that is not on the GPU")
+        T, cols = q.shape
+        dt = q.dtype
+        if not (cols == n_heads * head_dim and out.shape == q.shape):
+            raise KernelError("attention: q and out must be [T, heads*head_dim]")
+        if not (dt == out.dtype == k_pages.dtype == v_pages.dtype and dt in _DT):
+            raise KernelError("attention: dtypes differ")
+        # what depends on the step and the cache group only (tables, work lists, the split of the key range, scratch memory) is
+        # checked and decided at the step's first layer and kept with the step's description
+        key = (n_heads, n_kv_heads, head_dim, page_size, id(block_tables), dt)
+        plan = meta.plans.get(key)
+        if plan is None:
+            _dev(block_tables, meta.positions, meta.token_seq)
+            _req(meta.positions.numel() == T and meta.token_seq.numel() == T, "attention: one position and request row per token")
+            _req(block_tables.dtype == torch.int32 and block_tables.dim() == 2 and block_tables.is_contiguous(), "attention: bad block tables")
+            _req(n_heads % n_kv_heads == 0, "attention: heads must be a multiple of kv heads")
+            mfma = (dt == torch.bfloat16 and self.use_mfma and self.mfma_attention_supports(head_dim, n_heads // n_kv_heads)
+                    and page_size & (page_size - 1) == 0)  # the matrix-core kernels index pages with shifts
+            if dt == torch.bfloat16 and self.use_mfma and not mfma:
+                self._warn_slow_attention(head_dim, n_heads // n_kv_heads, page_size)
+            splits, ws, lib = 1, None, None
+            if mfma:
+                splits = self.decode_splits(meta, n_heads, n_kv_heads)
+                need = self.lib.lev_attention_mfma_workspace(meta.n_decode, splits, n_heads, n_kv_heads, head_dim) if splits > 1 else 0
+                ws = meta.workspace(need, q.device)
+                lib = self._unit(_build.attention_unit(head_dim))
+            plan = meta.plans[key] = (mfma, splits, ws, _ptr(ws), lib, _ptr(block_tables), block_tables.shape[1], _ptr(meta.positions),
+                                      _ptr(meta.token_seq), _ptr(meta.prefill_tiles), _ptr(meta.decode_tokens), block_tables)
+        mfma, splits, _ws, ws_ptr, lib, bt_ptr, bt_width, pos_ptr, seq_ptr, tiles_ptr, decode_ptr, _bt = plan
+        w = int(window) if window else 0
+        cap = float(softcap) if softcap else 0.0
+        bias_len = 0
+        if score_bias is not None:
+            if not (score_bias.is_cuda and score_bias.dtype == torch.float32 and score_bias.dim() == 2 and score_bias.shape[0] == n_heads
+                    and score_bias.is_contiguous() and score_bias.shape[1] >= 1):
+                raise KernelError("attention: the score bias must be a contiguous float32 table [heads, distances] on the GPU")
+            bias_len = score_bias.shape[1]
+        qs, os_ = _rows(q, "attention: q"), _rows(out, "attention: out")
+        kvs = 0
+        if k_new is not None:
+            fusable = mfma and meta.n_prefill_tiles == 0 and meta.n_decode == T
+            if not fusable:
+                return False
+            _dev(k_new, v_new, dest)
+            _req(k_new.shape == v_new.shape == (T, n_kv_heads * head_dim) and k_new.dtype == v_new.dtype == dt,
+                 "attention: new keys and values must be [T, kv_heads*head_dim] of the compute dtype")
+            _req(dest is not None and dest.dtype == torch.int32 and dest.numel() == T, "attention: one int32 destination per token")
+            kvs = _rows(k_new, "attention: k_new")
+            _req(kvs == _rows(v_new, "attention: v_new"), "attention: new keys and values must share a row stride")
+        if mfma:
+            self._check(lib.lev_attention_mfma(
+                _ptr(q), qs, _ptr(out), os_, _ptr(k_pages), _ptr(v_pages), pos_ptr, seq_ptr, bt_ptr, bt_width, tiles_ptr,
+                meta.n_prefill_tiles, decode_ptr, meta.n_decode, _ptr(k_new), _ptr(v_new), kvs,
+                _ptr(dest) if k_new is not None else None, ws_ptr, n_heads, n_kv_heads, head_dim, page_size,
+                splits, float(scale), w, cap, _ptr(score_bias), bias_len, self._s()))
+            return k_new is not None
+        self._check(self.lib.lev_attention_simple(
+            _ptr(q), qs, _ptr(out), os_, _ptr(k_pages), _ptr(v_pages), pos_ptr, seq_ptr, bt_ptr, bt_width, T, n_heads, n_kv_heads,
+            head_dim, page_size, float(scale), w, _DT[dt], cap, _ptr(score_bias), bias_len, self._s()))
+        return False
+
     @staticmethod
     def decode_splits(meta, n_heads: int, n_kv_heads: int) -> int:
         """Into how many key ranges a single-token query is split so that the chip is filled."""

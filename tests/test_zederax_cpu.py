@@ -161,3 +161,11 @@ def test_windowed_layers_give_pages_back_and_take_used_ones(tmp_path):
     cache.close(a)
     cache.close(b)
     cache.check_invariants()
+
+
+def test_the_hip_library_offers_every_launcher_that_its_stand_in_has():
+    from levanter_amd.kernels.library import HipKernels
+
+    missing = [n for n in dir(EmulatedKernels) if not n.startswith("_") and callable(getattr(EmulatedKernels, n))
+               and n not in ("k_view", "v_view", "gather_kv") and not hasattr(HipKernels, n)]
+    assert not missing, missing
