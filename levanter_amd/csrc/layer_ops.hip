@@ -54,6 +54,87 @@ extern "C" int lev_head_prepare(void* qk, long qk_stride, int n_norm, int hd, fl
 }
 
 // ------------------------------------------------------------------------------------------
+// The same for steps of single tokens, with the write into the cache's pages in the same kernel: one wave per (token,
+// item); items are the H query heads (normalised in place), the G key heads (normalised, written to the key pages
+// [page][G][hd/8][PS][8]) and the G value heads (blended, written to the value pages [page][G][vd][PS]). dest[t] =
+// page * PS + offset, negative for a token that is written nowhere. normalise == 0: queries and keys stay as they are.
+template <typename T>
+__global__ void __launch_bounds__(64)
+head_prepare_write_kernel(T* __restrict__ q, long q_stride, int H, const T* __restrict__ k, long k_stride, const T* __restrict__ v,
+                          long v_stride, const T* __restrict__ v_first, long vf_stride, const float* __restrict__ lambda, int G, int hd,
+                          int vd, float eps, int normalise, T* __restrict__ k_pages, T* __restrict__ v_pages,
+                          const int* __restrict__ dest, int PS) {
+  const int t = blockIdx.x, item = blockIdx.y, lane = threadIdx.x;
+  if (item < H + G) {
+    const bool is_q = item < H;
+    const T* row = is_q ? q + (size_t)t * q_stride + (size_t)item * hd : k + (size_t)t * k_stride + (size_t)(item - H) * hd;
+    float r = 1.0f;
+    if (normalise) {
+      float ss = 0.f;
+      for (int d = lane; d < hd; d += 64) {
+        const float x = to_float<T>(row[d]);
+        ss = fmaf(x, x, ss);
+      }
+      ss = wave_sum(ss);
+      r = 1.0f / sqrtf(ss / (float)hd + eps);
+    }
+    if (is_q) {
+      if (normalise) {
+        T* qrow = q + (size_t)t * q_stride + (size_t)item * hd;
+        for (int d = lane; d < hd; d += 64) qrow[d] = from_float<T>(to_float<T>(qrow[d]) * r);
+      }
+      return;
+    }
+    const int dst = dest[t];
+    if (dst < 0) return;
+    const int page = dst / PS, off = dst % PS;
+    T* kd = k_pages + ((size_t)page * G + (item - H)) * (size_t)hd * PS;
+    for (int d = lane; d < hd; d += 64) {
+      const float x = to_float<T>(row[d]);
+      kd[((size_t)(d >> 3) * PS + off) * 8 + (d & 7)] = normalise ? from_float<T>(x * r) : row[d];
+    }
+  } else {
+    const int c = item - H - G;
+    const int dst = dest[t];
+    if (dst < 0) return;
+    const int page = dst / PS, off = dst % PS;
+    const T* row = v + (size_t)t * v_stride + (size_t)c * vd;
+    T* vdst = v_pages + ((size_t)page * G + c) * (size_t)vd * PS + off;
+    if (v_first) {
+      const float lam = *lambda;
+      const T* first = v_first + (size_t)t * vf_stride + (size_t)c * vd;
+      for (int d = lane; d < vd; d += 64)
+        vdst[(size_t)d * PS] = from_float<T>((1.0f - lam) * to_float<T>(row[d]) + lam * to_float<T>(first[d]));
+    } else {
+      for (int d = lane; d < vd; d += 64) vdst[(size_t)d * PS] = row[d];
+    }
+  }
+}
+
+extern "C" int lev_head_prepare_write(void* q, long q_stride, int H, const void* k, long k_stride, const void* v, long v_stride,
+                                      const void* v_first, long vf_stride, const float* lambda, int G, int hd, int vd, float eps,
+                                      int normalise, void* k_pages, void* v_pages, const int* dest, int PS, int T, int dtype,
+                                      hipStream_t stream) {
+  LEV_REQUIRE(T >= 0 && H > 0 && G > 0 && hd > 0 && hd % 8 == 0 && vd > 0, "head_prepare_write: bad sizes T=%d heads=%d/%d sizes=%d/%d", T, H, G, hd, vd);
+  LEV_REQUIRE(q && k && v && k_pages && v_pages && dest, "head_prepare_write: a tensor is missing");
+  LEV_REQUIRE(!v_first || lambda, "head_prepare_write: values to blend need the weight");
+  LEV_REQUIRE(PS > 0 && PS % 16 == 0, "head_prepare_write: page_size=%d must be a multiple of 16", PS);
+  LEV_REQUIRE(H + 2 * G <= 65535, "head_prepare_write: too many heads (%d)", H + 2 * G);
+  LEV_REQUIRE(dtype == LEV_F32 || dtype == LEV_BF16, "head_prepare_write: unknown dtype %d", dtype);
+  if (T == 0) return 0;
+  dim3 grid(T, H + 2 * G);
+  if (dtype == LEV_F32)
+    head_prepare_write_kernel<float><<<grid, 64, 0, stream>>>((float*)q, q_stride, H, (const float*)k, k_stride, (const float*)v, v_stride,
+                                                             (const float*)v_first, vf_stride, lambda, G, hd, vd, eps, normalise,
+                                                             (float*)k_pages, (float*)v_pages, dest, PS);
+  else
+    head_prepare_write_kernel<bf16_t><<<grid, 64, 0, stream>>>((bf16_t*)q, q_stride, H, (const bf16_t*)k, k_stride, (const bf16_t*)v,
+                                                              v_stride, (const bf16_t*)v_first, vf_stride, lambda, G, hd, vd, eps,
+                                                              normalise, (bf16_t*)k_pages, (bf16_t*)v_pages, dest, PS);
+  return lev_check_launch("head_prepare_write");
+}
+
+// ------------------------------------------------------------------------------------------
 // out = c0 z / rms(z) + c1 z^2 / rms(z^2) + c2 z^3 / rms(z^3) + c3 over a row of F values, rms(u) = sqrt(mean(u^2) + eps).
 // One block per row; the row is read twice (statistics, then the output), the second time from the cache. `out` may be `z`.
 template <typename T, int NT>
@@ -178,4 +259,51 @@ extern "C" int lev_stream_average(float* streams, float* x, const float* w, int 
   LEV_REQUIRE(blocks <= 0x7fffffffL, "stream_average: too many elements (%ld)", count);
   stream_average_kernel<<<(unsigned)blocks, 256, 0, stream>>>(streams, x, w, n, count, vec);
   return lev_check_launch("stream_average");
+}
+
+// ------------------------------------------------------------------------------------------
+// The weighted sum above and the RMS norm that reads it, in one kernel: one block per output row keeps the summed row in
+// LDS between the statistics and the output. rows == null: every row, the sum is stored to x and the layer's result to
+// streams[n-1] exactly as stream_average does (the same additions in the same order). rows != null: output row r is the
+// norm of summed row rows[r]; nothing is stored (a selection may name a row twice, and nobody reads x after it).
+template <typename TO, int NT>
+__global__ void __launch_bounds__(NT)
+norm_average_kernel(float* __restrict__ streams, float* __restrict__ x, const float* __restrict__ w, int n, long count,
+                    const float* __restrict__ nw, TO* __restrict__ out, const int* __restrict__ rows, int D, float eps) {
+  extern __shared__ __attribute__((aligned(16))) float na_row[];
+  __shared__ float red[NT / 64];
+  const int r = blockIdx.x;
+  const long base = (long)(rows ? rows[r] : r) * D;
+  const bool store = rows == nullptr;
+  float ss = 0.f;
+  for (int d = threadIdx.x; d < D; d += NT) {
+    const float cur = x[base + d];
+    float s = 0.f;
+    for (int j = 0; j < n - 1; ++j) s = fmaf(w[j], streams[(size_t)j * count + base + d], s);
+    s = fmaf(w[n - 1], cur, s);
+    if (store) {
+      streams[(size_t)(n - 1) * count + base + d] = cur;
+      x[base + d] = s;
+    }
+    na_row[d] = s;
+    ss = fmaf(s, s, ss);
+  }
+  ss = block_sum<NT>(ss, red);
+  const float rinv = 1.0f / sqrtf(ss / (float)D + eps);
+  for (int d = threadIdx.x; d < D; d += NT) out[(size_t)r * D + d] = from_float<TO>(na_row[d] * rinv * nw[d]);
+}
+
+extern "C" int lev_norm_average(float* streams, float* x, const float* w, int n, long count, const float* norm_weight, void* out,
+                                const int* rows, int n_rows, int D, float eps, int out_dtype, hipStream_t stream) {
+  LEV_REQUIRE(n >= 1 && D > 0 && count >= 0 && count % D == 0 && streams && x && w && norm_weight && out, "norm_average: bad arguments n=%d D=%d", n, D);
+  LEV_REQUIRE((size_t)D * sizeof(float) <= 64 * 1024, "norm_average: rows of %d floats do not fit the LDS", D);
+  LEV_REQUIRE(out_dtype == LEV_F32 || out_dtype == LEV_BF16, "norm_average: unknown dtype %d", out_dtype);
+  LEV_REQUIRE(rows || (long)n_rows * D == count, "norm_average: without a selection every row is normalised");
+  if (n_rows == 0) return 0;
+  const size_t lds = (size_t)D * sizeof(float);
+  if (out_dtype == LEV_F32)
+    norm_average_kernel<float, 256><<<n_rows, 256, lds, stream>>>(streams, x, w, n, count, norm_weight, (float*)out, rows, D, eps);
+  else
+    norm_average_kernel<bf16_t, 256><<<n_rows, 256, lds, stream>>>(streams, x, w, n, count, norm_weight, (bf16_t*)out, rows, D, eps);
+  return lev_check_launch("norm_average");
 }

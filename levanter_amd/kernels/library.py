@@ -40,6 +40,17 @@ class PendingSum:
         self.out, self.workspace, self.n_ranges, self.bias, self.ldo = out, workspace, n_ranges, bias, ldo
 
 
+class PendingAverage:
+    """A weighted sum of residual streams that has not been computed yet (``HipKernels.stream_average(..., defer=True)``):
+    ``out`` (float32 ``[T, D]``) still holds the layer's own result. ``HipKernels.norm`` computes the sum inside the norm
+    that reads it; ``HipKernels.finish`` runs it by itself. Nothing else may read ``out`` before one of the two."""
+
+    __slots__ = ("out", "streams", "weights", "n")
+
+    def __init__(self, out, streams, weights, n):
+        self.out, self.streams, self.weights, self.n = out, streams, weights, n
+
+
 def _ptr(t: Optional[torch.Tensor]):
     """A tensor's address as ctypes takes it for a ``c_void_p`` parameter: a plain integer, or None."""
     return None if t is None else t.data_ptr()
@@ -206,7 +217,14 @@ class HipKernels:
             _req(n == x.shape[0], "norm: out must have as many rows as x")
         else:
             _req(rows.dtype == torch.int32 and rows.numel() == n, "norm: rows must be int32, one per output row")
-        if pending is not None:
+        if isinstance(pending, PendingAverage):
+            _req(pending.out is x, "norm: the unfinished sum belongs to another tensor")
+            if rms and bias is None and D * 4 <= 65536:
+                self._check(self.lib.lev_norm_average(_ptr(pending.streams), _ptr(x), _ptr(pending.weights), pending.n, x.numel(), _ptr(weight),
+                                                      _ptr(out), _ptr(rows), n, D, float(eps), _DT[out.dtype], self._s()))
+                return
+            self.finish(pending)
+        elif pending is not None:
             _req(pending.out is x and pending.ldo == D, "norm: the unfinished product belongs to another tensor")
             rc = self.lib.lev_norm_pending(_ptr(x), _ptr(pending.workspace), pending.n_ranges, _ptr(pending.bias), _ptr(weight), _ptr(bias),
                                            _ptr(out), _ptr(rows), n, x.shape[0], D, float(eps), int(rms), _DT[out.dtype], self._s())
@@ -240,7 +258,10 @@ class HipKernels:
         return new
 
     def finish(self, pending: PendingSum) -> None:
-        """Finish a product that ``linear(..., may_leave_pending=True)`` left unfinished."""
+        """Finish a product that ``linear(..., may_leave_pending=True)`` left unfinished, or a deferred sum of streams."""
+        if isinstance(pending, PendingAverage):
+            self.stream_average(pending.streams, pending.out, pending.weights, pending.n)
+            return
         x = pending.out
         self._check(self._unit("gemm_mfma").lev_linear_mfma_finish(_ptr(pending.workspace), _ptr(pending.bias), _ptr(x), pending.ldo, _ptr(x),
                                                                    pending.ldo, x.shape[0], x.shape[1], pending.n_ranges, 0, _DT[torch.float32],
@@ -378,6 +399,30 @@ class HipKernels:
                                               vs, _ptr(v_first) if n_blend else None, fs, int(n_blend), int(value_dim),
                                               _ptr(blend) if n_blend else None, T, _DT[dt], self._s()))
 
+    def head_prepare_write(self, q, k, v, k_pages, v_pages, dest, n_heads: int, n_kv_heads: int, head_dim: int, value_dim: int,
+                           page_size: int, eps: Optional[float], v_first=None, blend=None) -> None:
+        """``head_prepare`` and ``kv_write`` in one kernel, for steps of single tokens: queries are normalised in place
+        (``eps`` None: not at all), keys are normalised and values blended (``v_first`` None: not) on their way into the pages;
+        ``k`` and ``v`` themselves stay as projected."""
+        _dev(q, k, v, k_pages, v_pages, dest, v_first, blend)
+        T, dt = q.shape[0], q.dtype
+        _req(dt in _DT and dt == k.dtype == v.dtype == k_pages.dtype == v_pages.dtype, "head_prepare_write: dtypes differ")
+        _req(q.shape == (T, n_heads * head_dim) and k.shape == (T, n_kv_heads * head_dim) and v.shape == (T, n_kv_heads * value_dim),
+             "head_prepare_write: q, k, v must be [T, heads*size]")
+        _req(dest.dtype == torch.int32 and dest.numel() == T, "head_prepare_write: one int32 destination per token")
+        n_elems = k_pages.numel()
+        _req(k_pages.is_contiguous() and v_pages.is_contiguous() and n_elems % (n_kv_heads * head_dim * page_size) == 0
+             and n_elems * value_dim == v_pages.numel() * head_dim, "head_prepare_write: page tensors must be contiguous and fit the sizes")
+        fs = 0
+        if v_first is not None:
+            _req(v_first.shape == v.shape and v_first.dtype == dt and blend is not None and blend.dtype == torch.float32 and blend.numel() == 1,
+                 "head_prepare_write: blending needs values of the same shape and one float32 weight")
+            fs = _rows(v_first, "head_prepare_write: v_first")
+        self._check(self.lib.lev_head_prepare_write(
+            _ptr(q), _rows(q, "head_prepare_write: q"), n_heads, _ptr(k), _rows(k, "head_prepare_write: k"), _ptr(v),
+            _rows(v, "head_prepare_write: v"), _ptr(v_first), fs, _ptr(blend) if v_first is not None else None, n_kv_heads, head_dim,
+            value_dim, float(eps or 0.0), int(eps is not None), _ptr(k_pages), _ptr(v_pages), _ptr(dest), page_size, T, _DT[dt], self._s()))
+
     def poly_norm(self, z, coefficients, eps: float, out) -> None:
         """out = c0 z/rms(z) + c1 z^2/rms(z^2) + c2 z^3/rms(z^3) + c3 per row, rms(u) = sqrt(mean(u^2) + eps); powers element
         by element, statistics in 32-bit. ``coefficients``: float32 [4] on the GPU."""
@@ -404,14 +449,18 @@ class HipKernels:
         self._check(self.lib.lev_head_talk(_ptr(o), _ptr(talk), _ptr(gate), gs, _ptr(out), _rows(out, "head_talk: out"), T, n_heads, n_kv_heads,
                                            nv, value_dim, _DT[out.dtype], self._s()))
 
-    def stream_average(self, streams, x, weights, n: int) -> None:
+    def stream_average(self, streams, x, weights, n: int, defer: bool = False) -> Optional[PendingAverage]:
         """``streams`` float32 [slots, T, D] holds earlier results in entries 0 .. n-2. ``x`` (float32 [T, D]) is kept as entry
-        n-1 and becomes ``sum_j weights[j] streams[j]``, j = 0 .. n-1 in that order."""
+        n-1 and becomes ``sum_j weights[j] streams[j]``, j = 0 .. n-1 in that order. ``defer``: nothing is launched; the
+        ``PendingAverage`` that comes back goes to the norm that reads ``x`` next (or to ``finish``)."""
         _dev(streams, x, weights)
         _req(x.dtype == streams.dtype == weights.dtype == torch.float32 and x.is_contiguous() and streams.is_contiguous(), "stream_average: contiguous float32 tensors")
         _req(streams.dim() == 3 and streams.shape[1:] == x.shape and 1 <= n <= streams.shape[0], "stream_average: streams must be [slots >= n, T, D]")
         _req(weights.numel() >= n and weights.is_contiguous(), "stream_average: one weight per stream")
+        if defer:
+            return PendingAverage(x, streams, weights, int(n))
         self._check(self.lib.lev_stream_average(_ptr(streams), _ptr(x), _ptr(weights), int(n), x.numel(), self._s()))
+        return None
 
     def attention_values(self, q, out, k_pages, v_pages, meta, *, n_heads: int, n_kv_heads: int, head_dim: int, value_dim: int,
                          all_value_heads: bool, page_size: int, scale: float, window: Optional[int], block_tables,

@@ -58,5 +58,10 @@ class PolyNormMlp(FeedForward):
 
     def forward(self, h: torch.Tensor, x: torch.Tensor, ctx: StepContext) -> None:
         z = self.up(h, ctx)
-        ctx.kernels.poly_norm(z, self.coefficients, self.eps, z)
+        self.activate(z, ctx, z)
         self.down(z, ctx, residual=x, final=True)
+
+    def activate(self, z: torch.Tensor, ctx: StepContext, out: torch.Tensor) -> None:
+        """What lies between the two products: ``z`` ``[T, inner_dim]`` -> ``out`` (may be ``z``; rows may be strided). A block
+        that runs ``up`` and ``down`` as parts of larger products calls this directly."""
+        ctx.kernels.poly_norm(z, self.coefficients, self.eps, out)

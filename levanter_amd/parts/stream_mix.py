@@ -35,6 +35,7 @@ class DepthWeightedAverage(StreamMix):
 
     def enter(self, x: torch.Tensor, ctx: StepContext) -> None:
         if self.index == 0:  # the embedding's output is the first of the results
+            ctx.settle()
             streams = torch.empty((self.n_runs + 1,) + tuple(x.shape), dtype=torch.float32, device=x.device)
             streams[0].copy_(x)
             ctx.shared[self.KEY] = streams
@@ -43,4 +44,6 @@ class DepthWeightedAverage(StreamMix):
         streams = ctx.shared.get(self.KEY)
         if streams is None or streams.shape[1:] != x.shape:
             raise RuntimeError("depth_weighted_average: the run with index 0 has not been through this step")
-        ctx.kernels.stream_average(streams, x, self.weights, self.index + 2)
+        ctx.settle()
+        # where the block allows it the sum is left to the norm that reads x next (the next layer's, or the one before the head)
+        ctx.pending = ctx.kernels.stream_average(streams, x, self.weights, self.index + 2, defer=bool(ctx.may_defer))

@@ -103,9 +103,16 @@ class TalkingHeadsAttention(Mixer):
         return PagedKv(self.n_kv_heads, self.head_dim, self.window, None if self.value_dim == self.head_dim else self.value_dim)
 
     def forward(self, h: torch.Tensor, x: torch.Tensor, ctx: StepContext, unit: CacheUnitView, writes_cache: bool) -> None:
+        a = ctx.empty(h.shape[0], self.n_heads * self.value_dim)
+        self.attend(self.proj(h, ctx), ctx, unit, writes_cache, a)
+        self.out(a, ctx, residual=x, final=True)
+
+    def attend(self, p: torch.Tensor, ctx: StepContext, unit: CacheUnitView, writes_cache: bool, a: torch.Tensor) -> None:
+        """Everything between the two products: ``p`` ``[T, q | k | v | gate (| columns of others)]`` is what ``proj`` gives for
+        the mixer's input, ``a`` ``[T, heads * value_dim]`` (rows may be strided) takes the gated heads that ``out`` reads. A
+        block that runs ``proj`` and ``out`` as parts of larger products calls this directly."""
         K = ctx.kernels
-        T = h.shape[0]
-        p = self.proj(h, ctx)  # [T, q | k | v | gate], compute dtype
+        T = p.shape[0]
         o = self.offsets
         q = p[:, :self.q_cols]
         k = p[:, o["k"]:o["k"] + self.k_cols]
@@ -118,19 +125,22 @@ class TalkingHeadsAttention(Mixer):
             v_first = ctx.shared.get(self.value_mix_key)
             if v_first is None or v_first.shape != v.shape:
                 raise RuntimeError("attention: no layer before this one has left values of this shape to blend with")
-        n_norm = self.n_heads + self.n_kv_heads if self.unit_norm_eps is not None else 0
-        if n_norm or v_first is not None:
-            K.head_prepare(p[:, :self.q_cols + self.k_cols], n_norm, self.head_dim, self.unit_norm_eps or 0.0, v=v, v_first=v_first,
-                           n_blend=self.n_kv_heads if v_first is not None else 0, value_dim=self.value_dim, blend=self.blend)
         g = unit.group
-        if writes_cache:
-            K.kv_write(k, v, unit.k_pages, unit.v_pages, g.dest, self.n_kv_heads, self.head_dim, g.page_size, value_dim=self.value_dim)
+        if writes_cache and ctx.attention.n_prefill_tiles == 0:
+            # a step of single tokens: unit norms, the blend and the write into the pages are one kernel
+            K.head_prepare_write(q, k, v, unit.k_pages, unit.v_pages, g.dest, self.n_heads, self.n_kv_heads, self.head_dim, self.value_dim,
+                                 g.page_size, self.unit_norm_eps, v_first=v_first, blend=self.blend)
+        else:
+            n_norm = self.n_heads + self.n_kv_heads if self.unit_norm_eps is not None else 0
+            if n_norm or v_first is not None:
+                K.head_prepare(p[:, :self.q_cols + self.k_cols], n_norm, self.head_dim, self.unit_norm_eps or 0.0, v=v, v_first=v_first,
+                               n_blend=self.n_kv_heads if v_first is not None else 0, value_dim=self.value_dim, blend=self.blend)
+            if writes_cache:  # keys and values of 16 tokens at a time, transposed through LDS
+                K.kv_write(k, v, unit.k_pages, unit.v_pages, g.dest, self.n_kv_heads, self.head_dim, g.page_size, value_dim=self.value_dim)
         nv = self.n_kv_heads if self.talk is not None else 1
-        w = torch.empty((T, self.n_heads, nv, self.value_dim), dtype=torch.float32, device=h.device)
+        w = torch.empty((T, self.n_heads, nv, self.value_dim), dtype=torch.float32, device=p.device)
         K.attention_values(q, w, unit.k_pages, unit.v_pages, ctx.attention, n_heads=self.n_heads, n_kv_heads=self.n_kv_heads,
                            head_dim=self.head_dim, value_dim=self.value_dim, all_value_heads=self.talk is not None,
                            page_size=g.page_size, scale=self.scale, window=self.window, block_tables=g.block_tables,
                            softcap=self.softcap, slopes=self.slopes)
-        a = ctx.empty(T, self.n_heads * self.value_dim)
         K.head_talk(w, self.talk, gate, a, self.n_heads, self.n_kv_heads, self.value_dim)
-        self.out(a, ctx, residual=x, final=True)

@@ -173,6 +173,16 @@ class EmulatedKernels:
             lam = float(blend.reshape(-1)[0])
             v.copy_(((1.0 - lam) * v.float() + lam * v_first.float()).to(v.dtype))
 
+    def head_prepare_write(self, q, k, v, k_pages, v_pages, dest, n_heads, n_kv_heads, head_dim, value_dim, page_size, eps, v_first=None,
+                           blend=None) -> None:
+        k, v = k.clone(), v.clone()
+        if eps is not None:
+            self.head_prepare(q, n_heads, head_dim, eps)
+            self.head_prepare(k, n_kv_heads, head_dim, eps)
+        if v_first is not None:
+            self.head_prepare(None, 0, 0, 0.0, v=v, v_first=v_first, n_blend=n_kv_heads, value_dim=value_dim, blend=blend)
+        self.kv_write(k, v, k_pages, v_pages, dest, n_kv_heads, head_dim, page_size, value_dim=value_dim)
+
     def poly_norm(self, z, coefficients, eps, out) -> None:
         u = z.float()
         c = [float(x) for x in coefficients]
@@ -194,7 +204,7 @@ class EmulatedKernels:
             a = a * torch.sigmoid(gate.float())[:, :, None]
         out.copy_(a.reshape(T, -1).to(out.dtype))
 
-    def stream_average(self, streams, x, weights, n) -> None:
+    def stream_average(self, streams, x, weights, n, defer=False) -> None:
         streams[n - 1].copy_(x)
         acc = torch.zeros_like(x)
         for j in range(n):

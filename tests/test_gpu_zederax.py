@@ -60,6 +60,53 @@ def test_unit_norm_of_heads_and_blend_of_values(dtype, shape):
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("shape", [(5, 3, 1, 24, 8), (9, 4, 2, 64, 128), (1, 2, 2, 8, 16)])
+@pytest.mark.parametrize("blend", [True, False])
+def test_single_tokens_are_prepared_and_written_by_one_kernel(dtype, shape, blend):
+    """Unit norms, the blend and the write into the pages in one kernel, against the plain functions, with a token that is
+    written nowhere; the pages hold what the two separate kernels write."""
+    from emulated_kernels import EmulatedKernels
+
+    T, H, G, dk, dv = shape
+    ps, n_pages = 16, 6
+    g = torch.Generator().manual_seed(T + dk)
+    q = as_bf16_numbers(torch.randn(T, H * dk, generator=g))
+    k = as_bf16_numbers(torch.randn(T, G * dk, generator=g))
+    v = as_bf16_numbers(torch.randn(T, G * dv, generator=g))
+    first = as_bf16_numbers(torch.randn(T, G * dv, generator=g))
+    lam = torch.tensor([0.625])
+    dest = (torch.randperm(n_pages * ps, generator=g)[:T]).to(torch.int32)
+    if T > 2:
+        dest[1] = -1
+    qd, kd, vd_, fd = (t.to(dtype).to(DEV) for t in (q, k, v, first))
+    kp = torch.zeros(n_pages, G * dk * ps, dtype=dtype, device=DEV)
+    vp = torch.zeros(n_pages, G * dv * ps, dtype=dtype, device=DEV)
+    K().head_prepare_write(qd, kd, vd_, kp, vp, dest.to(DEV), H, G, dk, dv, ps, 1e-5, v_first=fd if blend else None, blend=lam.to(DEV) if blend else None)
+    want_q = Z.unit_rms(q.view(T, H, dk), 1e-5).reshape(T, -1)
+    want_k = Z.unit_rms(k.view(T, G, dk), 1e-5)
+    want_v = Z.blend_values(v, first if blend else None, lam.double()).view(T, G, dv)
+    torch.testing.assert_close(qd.cpu().double(), want_q, **tol(dtype))
+    kv = EmulatedKernels.k_view(kp.cpu().double(), G, dk, ps)
+    vv = EmulatedKernels.v_view(vp.cpu().double(), G, dv, ps)
+    for t in range(T):
+        d = int(dest[t])
+        if d < 0:
+            continue
+        torch.testing.assert_close(kv[d // ps, :, :, d % ps, :].reshape(G, dk), want_k[t], **tol(dtype))
+        torch.testing.assert_close(vv[d // ps, :, :, d % ps], want_v[t], **tol(dtype))
+    written = sum(1 for t in range(T) if int(dest[t]) >= 0)
+    assert int((kp != 0).sum()) <= written * G * dk and int((vp != 0).sum()) <= written * G * dv  # nothing else is touched
+    # the two separate kernels leave the same bits
+    q2, k2, v2 = (t.to(dtype).to(DEV) for t in (q, k, v))
+    qk = torch.cat([q2, k2], 1)
+    K().head_prepare(qk, H + G, dk, 1e-5, v=v2 if blend else None, v_first=fd if blend else None, n_blend=G if blend else 0, value_dim=dv,
+                     blend=lam.to(DEV) if blend else None)
+    kp2, vp2 = torch.zeros_like(kp), torch.zeros_like(vp)
+    K().kv_write(qk[:, H * dk:], v2, kp2, vp2, dest.to(DEV), G, dk, ps, value_dim=dv)
+    assert torch.equal(kp, kp2) and torch.equal(vp, vp2) and torch.equal(qd, qk[:, :H * dk])
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("T,F", [(3, 40), (70, 1000), (2, 8200)])
 def test_polynomial_activation_with_normed_powers(dtype, T, F):
     g = torch.Generator().manual_seed(F)
@@ -89,6 +136,36 @@ def test_weighted_sum_of_all_results_so_far(T, D):
         want = Z.depth_average([r.double() for r in results[:i + 2]], w.double())
         torch.testing.assert_close(x.cpu().double(), want, rtol=1e-5, atol=1e-5)
         assert torch.equal(streams[i + 1].cpu(), results[i + 1])
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("T,D", [(7, 64), (3, 30), (40, 1000)])
+def test_weighted_sum_inside_the_norm_that_reads_it(dtype, T, D):
+    """The deferred sum: computed by the norm's kernel, stored as the separate kernel stores it; with a selection of rows
+    (one named twice) only the normed rows come out."""
+    g = torch.Generator().manual_seed(D + 1)
+    n = 4
+    results = [torch.randn(T, D, generator=g) for _ in range(n)]
+    w, nw = torch.randn(n, generator=g), 1 + 0.2 * torch.randn(D, generator=g)
+    want_x = Z.depth_average([r.double() for r in results], w.double())
+    want_h = Z.rms_norm(want_x, nw.double(), 1e-5)
+    for rows in (None, torch.tensor([T - 1, 0, T - 1], dtype=torch.int32)):
+        streams = torch.zeros(n + 2, T, D, device=DEV)
+        for j in range(n - 1):
+            streams[j] = results[j].to(DEV)
+        x = results[n - 1].clone().to(DEV)
+        pending = K().stream_average(streams, x, w.to(DEV), n, defer=True)
+        assert pending is not None and torch.equal(x.cpu(), results[n - 1])  # nothing has run yet
+        out = torch.empty(T if rows is None else 3, D, dtype=dtype, device=DEV)
+        K().norm(x, nw.to(DEV), None, 1e-5, out, rows=None if rows is None else rows.to(DEV), rms=True, pending=pending)
+        torch.testing.assert_close(out.cpu().double(), want_h if rows is None else want_h[rows.long()], **tol(dtype))
+        if rows is None:
+            torch.testing.assert_close(x.cpu().double(), want_x, rtol=1e-5, atol=1e-5)
+            assert torch.equal(streams[n - 1].cpu(), results[n - 1])
+            # and the same bits as the kernel that only sums
+            x2 = results[n - 1].clone().to(DEV)
+            K().stream_average(streams, x2, w.to(DEV), n)
+            assert torch.equal(x2, x)
 
 
 def run_attention(dtype, H, G, dk, dv, runs, window, cap, scale, q, k, v, talk, gate, ps=16, seed=0):
