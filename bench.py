@@ -60,6 +60,8 @@ def main() -> int:
                          "through InferenceEngine.generate; they print their own line. zederax: prefill and decode rates of Zederax "
                          "layers at a few sizes beside GPT-2 layers of the same width, heads and inner width; its own line")
     ap.add_argument("--sizes", default="1k,2k,4k", help="with --workload zederax: which of the sizes 1k, 2k, 4k to run")
+    ap.add_argument("--batches", default="1,8,64", help="with --workload zederax: decode batch sizes to time ('' for none)")
+    ap.add_argument("--no-prefill", action="store_true", help="with --workload zederax: skip the 2,048-token prompt")
     ap.add_argument("--arch", default="both", choices=["both", "zederax", "gpt2"], help="with --workload zederax: one architecture only (for profiling)")
     args = ap.parse_args()
     if args.gpus != 1:
@@ -331,7 +333,7 @@ def zederax_workload(args) -> int:
 
     ps, prompt_len, V = 16, 512, ZEDERAX_VOCAB
     steps, warmup = min(args.steps, 128), args.warmup
-    batches = (1, 8, 64)
+    batches = tuple(int(b) for b in args.batches.split(",") if b)
     ctx_end = prompt_len + 64 + warmup + steps + 16
     pages_per_seq = (max(ctx_end, 2048) + ps - 1) // ps
 
@@ -340,13 +342,14 @@ def zederax_workload(args) -> int:
         return [torch.randint(0, V, (n,), generator=g).tolist() for _ in range(batch)]
 
     def measure(raw):
-        ecfg = InferenceEngineConfig(max_pages=max(batches) * ((ctx_end + ps - 1) // ps) + pages_per_seq, max_seqs=max(batches), page_size=ps,
+        most = max(batches, default=1)
+        ecfg = InferenceEngineConfig(max_pages=most * ((ctx_end + ps - 1) // ps) + pages_per_seq, max_seqs=most, page_size=ps,
                                      max_pages_per_seq=pages_per_seq, compute_dtype=args.dtype, max_prefill_size=2048,
-                                     max_seqs_in_prefill=max(batches))
+                                     max_seqs_in_prefill=most)
         engine = InferenceEngine.from_config(LmConfig.from_dict(raw), seed=0, config=ecfg)
         out = {"weights_gb": round(engine.model.weight_bytes() / 1e9, 3)}
         times = []
-        for rep in range(4):
+        for rep in range(0 if args.no_prefill else 4):
             engine.reset()
             engine.enqueue_requests([Request(prompt_tokens=prompts(1, 2048, 50 + rep)[0], request_id=rep, max_new_tokens=1)])
             torch.cuda.synchronize()
@@ -355,7 +358,9 @@ def zederax_workload(args) -> int:
             torch.cuda.synchronize()
             if rep > 0:
                 times.append(time.perf_counter() - t)
-        out["prefill_2048_tok_s"] = round(2048 / sorted(times)[len(times) // 2], 1)
+        if times:
+            out["prefill_2048_tok_s"] = round(2048 / sorted(times)[len(times) // 2], 1)
+            out["prefill_2048_ms"] = round(sorted(times)[len(times) // 2] * 1e3, 3)
         for b in batches:
             engine.reset()
             reqs = [Request(prompt_tokens=p, request_id=i, max_new_tokens=64 + warmup + steps + 8, temperature=0.0)

@@ -10,11 +10,13 @@
 // a block of 64, so that lane group g = l/16 holds the weights of the keys 32u + 8g .. +7 in its two tiles.
 //
 // One wave owns 16 columns that share a request and a key/value head:
-//   * a run of several tokens: 16 consecutive query tokens of one query head;
-//   * a single token: the query heads of one key/value head (up to 16 at a time).
-// It walks the keys in blocks of 64 (operands go from the pages straight into registers), keeps a running maximum and sum
-// per column, and applies the weights to the values of `nvc` value heads (blockIdx.z picks which): its own one, or, for
-// layers that mix the weights over the heads afterwards, every key/value head in turn.
+//   * a run of several tokens: 16 consecutive query tokens of one query head; the 8 waves of a workgroup are a tile of up
+//     to 128 tokens and share every block of keys and values through LDS (attention_values_mfma_runs_kernel);
+//   * a single token: the query heads of one key/value head (up to 16 at a time); operands go from the pages straight
+//     into registers, and a token's keys may be split over several waves whose results a second kernel merges.
+// A wave walks the keys in blocks of 64, keeps a running maximum and sum per column, and applies the weights to the
+// values of up to NVC value heads (blockIdx.z picks which): its own one, or, for layers that mix the weights over the
+// heads afterwards, every key/value head in turn.
 //
 //   score(t, key) = cap(scale * q . k) - slope[h] * (position(t) - position(key)),  cap(s) = softcap * tanh(s / softcap)
 //   out [T][H][NV][VD] float32, as attention_values.hip writes it.
@@ -60,7 +62,8 @@ __global__ void __launch_bounds__(64)
 attention_values_mfma_kernel(const bf16_t* __restrict__ q, long q_stride, float* __restrict__ out, const bf16_t* __restrict__ k_pages,
                              const bf16_t* __restrict__ v_pages, const int* __restrict__ positions, const int* __restrict__ token_seq,
                              const int* __restrict__ block_tables, int bt_stride, const int* __restrict__ work, int H, int KVH, int NV,
-                             int PS, float scale, int window, float softcap, const float* __restrict__ slopes) {
+                             int PS, float scale, int window, float softcap, const float* __restrict__ slopes, int splits,
+                             float* __restrict__ part_o, float* __restrict__ part_ml) {
   const int lane = threadIdx.x, col = lane & 15, g = lane >> 4;
   const int group = H / KVH;
   int tok = 0, head = 0, kvh = 0;
@@ -71,7 +74,7 @@ attention_values_mfma_kernel(const bf16_t* __restrict__ q, long q_stride, float*
     const int c = (blockIdx.y % col_sets) * 16 + col;
     valid = c < group;
     head = kvh * group + (valid ? c : 0);
-    tok = work[blockIdx.x];
+    tok = work[blockIdx.x / splits];
   } else {
     const int tile = blockIdx.x / SUB_TILES, sub = blockIdx.x % SUB_TILES;
     const int first = work[2 * tile], n = work[2 * tile + 1];
@@ -111,7 +114,14 @@ attention_values_mfma_kernel(const bf16_t* __restrict__ q, long q_stride, float*
   constexpr float LOG2E = 1.4426950408889634f;
   const size_t k_head = (size_t)HD * PS, v_head = (size_t)VD * PS;
 
-  for (int key0 = (lo_min / 64) * 64; key0 <= p_max; key0 += 64) {
+  // a single token's keys may be split over `splits` waves (blockIdx.x % splits): each takes a run of whole blocks
+  int key_first = (lo_min / 64) * 64, key_last = p_max;
+  if (SINGLE && splits > 1) {
+    const int n_blocks = p_max / 64 - lo_min / 64 + 1, per = (n_blocks + splits - 1) / splits, z = blockIdx.x % splits;
+    key_first += z * per * 64;
+    key_last = min(p_max, key_first + per * 64 - 1);
+  }
+  for (int key0 = key_first; key0 <= key_last; key0 += 64) {
     // pages of this lane's two groups of 8 keys (32u + 8g .. +7): for the mask and for the values
     int pgv[2];
 #pragma unroll
@@ -200,6 +210,22 @@ attention_values_mfma_kernel(const bf16_t* __restrict__ q, long q_stride, float*
   l += __shfl_xor(l, 16, 64);
   l += __shfl_xor(l, 32, 64);
   if (!valid) return;
+  if (SINGLE && splits > 1) {  // unnormalised sums, the maximum and the sum of weights: merged by the kernel below
+    const size_t slot = ((size_t)blockIdx.x * H + head);  // (token index, split) major, then head
+    if (g == 0 && blockIdx.z == 0) {
+      part_ml[2 * slot] = m;
+      part_ml[2 * slot + 1] = l;
+    }
+#pragma unroll
+    for (int c = 0; c < NVC; ++c) {
+      if (c < n_c) {
+        float* ob = part_o + (slot * NV + (NV == 1 ? 0 : c0 + c)) * VD;
+#pragma unroll
+        for (int dt = 0; dt < NDT; ++dt) *reinterpret_cast<f32x4*>(ob + 16 * dt + 4 * g) = o[c][dt];
+      }
+    }
+    return;
+  }
   const float inv = l > 0.f ? 1.0f / l : 0.f;
 #pragma unroll
   for (int c = 0; c < NVC; ++c) {
@@ -211,16 +237,238 @@ attention_values_mfma_kernel(const bf16_t* __restrict__ q, long q_stride, float*
   }
 }
 
+// Runs of several tokens: one workgroup of PF_WAVES waves per (tile of up to PF_ROWS consecutive query tokens, query head,
+// set of value heads). The keys and values of a block of 64 positions are staged once for all waves: global -> registers
+// (requested one block ahead, while the block before is computed) -> LDS, keys as [HD/8][64][8], values transposed as
+// [value head][VD][64 + 8] with everything beyond the last written key made zero on the way.
+#define VS_STRIDE 72
+#define K_STAGE ((HD * 8 + PF_THREADS - 1) / PF_THREADS)        // 16-byte chunks of a key block per thread
+#define V_STAGE ((NVC * VD * 8 + PF_THREADS - 1) / PF_THREADS)  // and of the value blocks
+
+__global__ void __launch_bounds__(PF_THREADS)
+attention_values_mfma_runs_kernel(const bf16_t* __restrict__ q, long q_stride, float* __restrict__ out, const bf16_t* __restrict__ k_pages,
+                                  const bf16_t* __restrict__ v_pages, const int* __restrict__ positions, const int* __restrict__ token_seq,
+                                  const int* __restrict__ block_tables, int bt_stride, const int* __restrict__ tiles, int H, int KVH, int NV,
+                                  int PS, float scale, int window, float softcap, const float* __restrict__ slopes) {
+  extern __shared__ __attribute__((aligned(16))) unsigned char av_smem[];
+  bf16_t* ks = reinterpret_cast<bf16_t*>(av_smem);  // [HD/8][64][8]
+  bf16_t* vs = ks + HD * 64;                        // [n_c][VD][VS_STRIDE]
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, col = lane & 15, g = lane >> 4;
+  const int first = tiles[2 * blockIdx.x], n = tiles[2 * blockIdx.x + 1];
+  if (n <= 0) return;  // the whole workgroup
+  const int head = blockIdx.y, group = H / KVH, kvh = head / group;
+  const bool active = wave * 16 < n;            // this wave has query rows
+  const bool valid = wave * 16 + col < n;       // this lane's column is one of them
+  const int tok = first + (valid ? wave * 16 + col : 0);
+  const int pos0 = positions[first];
+  const int pos = pos0 + (tok - first);         // a run's tokens stand at consecutive positions
+  const int lo = window > 0 ? max(0, pos - window + 1) : 0;
+  const int p_max_wg = pos0 + n - 1, lo_wg = window > 0 ? max(0, pos0 - window + 1) : 0;
+  const int p_max = min(p_max_wg, pos0 + wave * 16 + 15);                                   // this wave's rows
+  const int lo_min = window > 0 ? max(0, pos0 + wave * 16 - window + 1) : 0;
+  const int* bt = block_tables + (size_t)token_seq[first] * bt_stride;
+  const float slope = slopes ? slopes[head] : 0.f;
+  const int c0 = NV == 1 ? kvh : blockIdx.z * NVC;
+  const int n_c = NV == 1 ? 1 : min(NVC, NV - blockIdx.z * NVC);
+
+  u32x4 qf[NKS];
+#pragma unroll
+  for (int s = 0; s < NKS; ++s) {
+    qf[s] = u32x4{0u, 0u, 0u, 0u};
+    if (valid && 32 * s + 8 * g < HD)
+      qf[s] = *reinterpret_cast<const u32x4*>(q + (size_t)tok * q_stride + (size_t)head * HD + 32 * s + 8 * g);
+  }
+  f32x4 o[NVC][NDT];
+#pragma unroll
+  for (int c = 0; c < NVC; ++c)
+#pragma unroll
+    for (int dt = 0; dt < NDT; ++dt) o[c][dt] = f32x4{0.f, 0.f, 0.f, 0.f};
+  float m = -INFINITY, l = 0.f;
+  constexpr float LOG2E = 1.4426950408889634f;
+  const size_t k_head = (size_t)HD * PS, v_head = (size_t)VD * PS;
+
+  u32x4 kst[K_STAGE], vst[V_STAGE];
+  // this thread's chunks of the block at key0, from the pages into registers
+  auto fetch = [&](int key0) {
+#pragma unroll
+    for (int i = 0; i < K_STAGE; ++i) {
+      const int ci = tid + PF_THREADS * i;  // (chunk of 8 dims, key)
+      kst[i] = u32x4{0u, 0u, 0u, 0u};
+      if (ci < HD * 8) {
+        const int kp = key0 + (ci & 63);
+        const int page = kp <= p_max_wg ? bt[kp / PS] : -1;
+        if (page >= 0) kst[i] = *reinterpret_cast<const u32x4*>(k_pages + ((size_t)page * KVH + kvh) * k_head + ((size_t)(ci >> 6) * PS + kp % PS) * 8);
+      }
+    }
+#pragma unroll
+    for (int i = 0; i < V_STAGE; ++i) {
+      const int ci = tid + PF_THREADS * i;  // (value head, dim, group of 8 keys)
+      vst[i] = u32x4{0u, 0u, 0u, 0u};
+      if (ci < n_c * VD * 8) {
+        const int kp = key0 + 8 * (ci & 7), row = ci >> 3;  // row = c * VD + dim
+        const int page = kp <= p_max_wg ? bt[kp / PS] : -1;
+        if (page >= 0) {
+          const u32x4 v = *reinterpret_cast<const u32x4*>(v_pages + ((size_t)page * KVH + c0 + row / VD) * v_head + (size_t)(row % VD) * PS + kp % PS);
+          vst[i] = first_keys(v, min(8, p_max_wg - kp + 1));
+        }
+      }
+    }
+  };
+  auto stage = [&]() {
+#pragma unroll
+    for (int i = 0; i < K_STAGE; ++i) {
+      const int ci = tid + PF_THREADS * i;
+      if (ci < HD * 8) *reinterpret_cast<u32x4*>(ks + (size_t)ci * 8) = kst[i];
+    }
+#pragma unroll
+    for (int i = 0; i < V_STAGE; ++i) {
+      const int ci = tid + PF_THREADS * i;
+      if (ci < n_c * VD * 8) *reinterpret_cast<u32x4*>(vs + (size_t)(ci >> 3) * VS_STRIDE + 8 * (ci & 7)) = vst[i];
+    }
+  };
+
+  const int key_begin = (lo_wg / 64) * 64;
+  fetch(key_begin);
+  for (int key0 = key_begin; key0 <= p_max_wg; key0 += 64) {
+    __syncthreads();  // the block before has been read by every wave
+    stage();
+    __syncthreads();
+    if (key0 + 64 <= p_max_wg) fetch(key0 + 64);
+    if (!active || key0 > p_max || key0 + 63 < lo_min) continue;  // none of this wave's rows sees a key of this block
+    int pgv[2];
+#pragma unroll
+    for (int u = 0; u < 2; ++u) {
+      const int kp = key0 + 32 * u + 8 * g;
+      pgv[u] = kp <= p_max ? bt[kp / PS] : -1;
+    }
+    f32x4 st[2][2];
+#pragma unroll
+    for (int u = 0; u < 2; ++u)
+#pragma unroll
+      for (int hh = 0; hh < 2; ++hh) {
+        const int key_row = 32 * u + 8 * (col >> 2) + 4 * hh + (col & 3);
+        f32x4 acc = f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int s = 0; s < NKS; ++s) {
+          u32x4 kf = u32x4{0u, 0u, 0u, 0u};
+          if (32 * s + 8 * g < HD) kf = *reinterpret_cast<const u32x4*>(ks + ((size_t)(4 * s + g) * 64 + key_row) * 8);
+          acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_bf16x8(kf), as_bf16x8(qf[s]), acc, 0, 0, 0);
+        }
+        st[u][hh] = acc;
+      }
+    float mx = -INFINITY;
+#pragma unroll
+    for (int u = 0; u < 2; ++u)
+#pragma unroll
+      for (int hh = 0; hh < 2; ++hh)
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+          const int kp = key0 + 32 * u + 8 * g + 4 * hh + r;
+          const bool ok = valid && kp <= pos && kp >= lo && pgv[u] >= 0;
+          float sc = st[u][hh][r] * scale;
+          if (softcap > 0.f) sc = softcap * fast_tanh(sc * __builtin_amdgcn_rcpf(softcap));
+          sc = (sc - slope * (float)(pos - kp)) * LOG2E;
+          sc = ok ? sc : -INFINITY;
+          st[u][hh][r] = sc;
+          mx = fmaxf(mx, sc);
+        }
+    mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
+    mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
+    const float m_new = fmaxf(m, mx);
+    const float m_use = m_new == -INFINITY ? 0.f : m_new;
+    const float corr = __builtin_amdgcn_exp2f(m - m_use);
+    m = m_new;
+    float psum = 0.f;
+    u32x4 pf[2];
+#pragma unroll
+    for (int u = 0; u < 2; ++u) {
+      float p[8];
+#pragma unroll
+      for (int hh = 0; hh < 2; ++hh)
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+          p[4 * hh + r] = __builtin_amdgcn_exp2f(st[u][hh][r] - m_use);
+          psum += p[4 * hh + r];
+        }
+#pragma unroll
+      for (int e = 0; e < 4; ++e) pf[u][e] = float2_to_bf16x2(p[2 * e], p[2 * e + 1]);
+    }
+    l = l * corr + psum;
+#pragma unroll
+    for (int c = 0; c < NVC; ++c) {
+      if (c < n_c) {
+#pragma unroll
+        for (int dt = 0; dt < NDT; ++dt) {
+          f32x4 acc = o[c][dt] * corr;
+#pragma unroll
+          for (int u = 0; u < 2; ++u) {
+            const u32x4 vf = *reinterpret_cast<const u32x4*>(vs + (size_t)(c * VD + 16 * dt + col) * VS_STRIDE + 32 * u + 8 * g);
+            acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_bf16x8(vf), as_bf16x8(pf[u]), acc, 0, 0, 0);
+          }
+          o[c][dt] = acc;
+        }
+      }
+    }
+  }
+  l += __shfl_xor(l, 16, 64);
+  l += __shfl_xor(l, 32, 64);
+  if (!valid) return;
+  const float inv = l > 0.f ? 1.0f / l : 0.f;
+#pragma unroll
+  for (int c = 0; c < NVC; ++c) {
+    if (c < n_c) {
+      float* ob = out + (((size_t)tok * H + head) * NV + (NV == 1 ? 0 : c0 + c)) * VD;
+#pragma unroll
+      for (int dt = 0; dt < NDT; ++dt) *reinterpret_cast<f32x4*>(ob + 16 * dt + 4 * g) = o[c][dt] * inv;
+    }
+  }
+}
+
+// Merges the splits of a single token's keys: out[tok][head] = sum_s 2^(m_s - M) o_s / sum_s 2^(m_s - M) l_s, in the order of s.
+__global__ void __launch_bounds__(64)
+attention_values_merge_kernel(const float* __restrict__ part_o, const float* __restrict__ part_ml, const int* __restrict__ singles,
+                              float* __restrict__ out, int H, int n_out, int splits) {
+  const int idx = blockIdx.x, head = blockIdx.y, lane = threadIdx.x;
+  // lane s holds split s's maximum and sum (at most 64 splits)
+  float ms = -INFINITY, ls = 0.f;
+  if (lane < splits) {
+    const size_t slot = ((size_t)idx * splits + lane) * H + head;
+    ms = part_ml[2 * slot];
+    ls = part_ml[2 * slot + 1];
+  }
+  const float M = wave_max(ms);
+  const float ws = __builtin_amdgcn_exp2f(ms - (M == -INFINITY ? 0.f : M));  // no keys: 0
+  float L = ws * ls;
+  // the sum in the order of the splits
+  float Lsum = 0.f;
+  for (int s = 0; s < splits; ++s) Lsum += __shfl(L, s, 64);
+  const float inv = Lsum > 0.f ? 1.0f / Lsum : 0.f;
+  float* o = out + ((size_t)singles[idx] * H + head) * n_out;
+  const float* po = part_o + ((size_t)idx * splits * H + head) * n_out;
+  for (int e = lane; e < n_out; e += 64) {
+    float acc = 0.f;
+#pragma unroll 4
+    for (int s = 0; s < splits; ++s) acc = fmaf(__shfl(ws, s, 64), po[(size_t)s * H * n_out + e], acc);
+    o[e] = acc * inv;
+  }
+}
+
+// bytes of scratch memory for n single tokens whose keys are split `splits` ways
+extern "C" long lev_attention_values_mfma_workspace(int n_singles, int splits, int H, int NV) {
+  return splits <= 1 ? 0 : (long)n_singles * splits * H * ((long)NV * VD + 2) * (long)sizeof(float);
+}
+
 extern "C" int lev_attention_values_mfma(const void* q, long q_stride, float* out, const void* k_pages, const void* v_pages,
                                          const int* positions, const int* token_seq, const int* block_tables, int bt_stride,
                                          const int* tiles, int n_tiles, const int* singles, int n_singles, int H, int KVH, int HD_,
                                          int VD_, int NV, int PS, float scale, int window, float softcap, const float* slopes,
-                                         hipStream_t stream) {
+                                         int splits, float* workspace, hipStream_t stream) {
   LEV_REQUIRE(HD_ == HD && VD_ == VD, "attention: this library was built for head sizes %d / %d, not %d / %d", HD, VD, HD_, VD_);
   LEV_REQUIRE(H > 0 && KVH > 0 && H % KVH == 0, "attention: bad head counts heads=%d kv_heads=%d", H, KVH);
   LEV_REQUIRE(NV == 1 || NV == KVH, "attention: %d value heads per query head (1 or kv_heads=%d)", NV, KVH);
   LEV_REQUIRE(PS > 0 && PS % 16 == 0, "attention: page_size=%d must be a multiple of 16", PS);
   LEV_REQUIRE(window >= 0 && softcap >= 0.f, "attention: window=%d and soft cap %g must not be negative", window, (double)softcap);
+  LEV_REQUIRE(splits >= 1 && splits <= 64 && (splits == 1 || workspace), "attention: %d splits (at most 64) need scratch memory", splits);
   LEV_REQUIRE(n_tiles >= 0 && n_singles >= 0 && (n_tiles == 0 || tiles) && (n_singles == 0 || singles), "attention: bad work lists");
   LEV_REQUIRE(((uintptr_t)q & 15) == 0 && q_stride % 8 == 0 && ((uintptr_t)k_pages & 15) == 0 && ((uintptr_t)v_pages & 15) == 0 &&
                   ((uintptr_t)out & 15) == 0,
@@ -228,19 +476,32 @@ extern "C" int lev_attention_values_mfma(const void* q, long q_stride, float* ou
   const int chunks = NV == 1 ? 1 : (NV + NVC - 1) / NVC;
   LEV_REQUIRE(H <= 65535 && chunks <= 65535, "attention: too many heads (%d)", H);
   if (n_tiles > 0) {
-    dim3 grid(n_tiles * SUB_TILES, H, chunks);
-    attention_values_mfma_kernel<false><<<grid, 64, 0, stream>>>((const bf16_t*)q, q_stride, out, (const bf16_t*)k_pages,
-                                                                (const bf16_t*)v_pages, positions, token_seq, block_tables, bt_stride,
-                                                                tiles, H, KVH, NV, PS, scale, window, softcap, slopes);
+    dim3 grid(n_tiles, H, chunks);
+    const size_t lds = ((size_t)HD * 64 + (size_t)(NV == 1 ? 1 : (NV < NVC ? NV : NVC)) * VD * VS_STRIDE) * sizeof(bf16_t);
+    if (lds <= 64 * 1024)
+      attention_values_mfma_runs_kernel<<<grid, PF_THREADS, lds, stream>>>((const bf16_t*)q, q_stride, out, (const bf16_t*)k_pages,
+                                                                         (const bf16_t*)v_pages, positions, token_seq, block_tables,
+                                                                         bt_stride, tiles, H, KVH, NV, PS, scale, window, softcap, slopes);
+    else  // the largest head sizes: every wave by itself, operands straight from the pages
+      attention_values_mfma_kernel<false><<<dim3(n_tiles * SUB_TILES, H, chunks), 64, 0, stream>>>(
+          (const bf16_t*)q, q_stride, out, (const bf16_t*)k_pages, (const bf16_t*)v_pages, positions, token_seq, block_tables, bt_stride,
+          tiles, H, KVH, NV, PS, scale, window, softcap, slopes, 1, nullptr, nullptr);
     if (lev_check_launch("attention_values_mfma (runs)")) return -1;
   }
   if (n_singles > 0) {
     const int group = H / KVH;
-    dim3 grid(n_singles, KVH * ((group + 15) / 16), chunks);
+    dim3 grid(n_singles * splits, KVH * ((group + 15) / 16), chunks);
+    float* part_o = workspace;
+    float* part_ml = splits > 1 ? workspace + (size_t)n_singles * splits * H * NV * VD : nullptr;
     attention_values_mfma_kernel<true><<<grid, 64, 0, stream>>>((const bf16_t*)q, q_stride, out, (const bf16_t*)k_pages,
                                                                (const bf16_t*)v_pages, positions, token_seq, block_tables, bt_stride,
-                                                               singles, H, KVH, NV, PS, scale, window, softcap, slopes);
+                                                               singles, H, KVH, NV, PS, scale, window, softcap, slopes, splits, part_o,
+                                                               part_ml);
     if (lev_check_launch("attention_values_mfma (single tokens)")) return -1;
+    if (splits > 1) {
+      attention_values_merge_kernel<<<dim3(n_singles, H), 64, 0, stream>>>(part_o, part_ml, singles, out, H, NV * VD, splits);
+      if (lev_check_launch("attention_values_mfma (merge)")) return -1;
+    }
   }
   return 0;
 }

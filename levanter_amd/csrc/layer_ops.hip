@@ -165,6 +165,73 @@ poly_norm_kernel(const T* z, long z_stride, T* out, long o_stride, const float* 
   }
 }
 
+// The same with the row in registers between the two passes: 16-byte loads, every load of the row in flight at once.
+// NCH chunks of 16 bytes per thread; rows of up to NT * NCH * (16 / sizeof(T)) values whose length is a multiple of a chunk.
+template <typename T, int NT, int NCH>
+__global__ void __launch_bounds__(NT)
+poly_norm_reg_kernel(const T* z, long z_stride, T* out, long o_stride, const float* __restrict__ coef, int F, float eps) {
+  typedef __attribute__((ext_vector_type(4))) uint32_t u32x4;
+  constexpr int E = 16 / (int)sizeof(T);  // values per chunk
+  __shared__ float red[NT / 64];
+  const T* row = z + (size_t)blockIdx.x * z_stride;
+  T* o = out + (size_t)blockIdx.x * o_stride;
+  const int n_chunks = F / E;
+  union Chunk { u32x4 raw; T v[E]; };
+  Chunk ch[NCH];
+#pragma unroll
+  for (int i = 0; i < NCH; ++i) {
+    const int c = threadIdx.x + NT * i;
+    ch[i].raw = u32x4{0u, 0u, 0u, 0u};
+    if (c < n_chunks) ch[i].raw = *reinterpret_cast<const u32x4*>(row + (size_t)c * E);
+  }
+  float s2 = 0.f, s4 = 0.f, s6 = 0.f;
+#pragma unroll
+  for (int i = 0; i < NCH; ++i)
+#pragma unroll
+    for (int e = 0; e < E; ++e) {
+      const float u = to_float<T>(ch[i].v[e]);
+      const float u2 = u * u, u3 = u2 * u;
+      s2 += u2;
+      s4 = fmaf(u2, u2, s4);
+      s6 = fmaf(u3, u3, s6);
+    }
+  s2 = block_sum<NT>(s2, red);
+  s4 = block_sum<NT>(s4, red);
+  s6 = block_sum<NT>(s6, red);
+  const float inv = 1.0f / (float)F;
+  const float r1 = coef[0] / sqrtf(s2 * inv + eps), r2 = coef[1] / sqrtf(s4 * inv + eps), r3 = coef[2] / sqrtf(s6 * inv + eps);
+  const float c3 = coef[3];
+#pragma unroll
+  for (int i = 0; i < NCH; ++i) {
+    const int c = threadIdx.x + NT * i;
+    if (c < n_chunks) {
+      Chunk w;
+#pragma unroll
+      for (int e = 0; e < E; ++e) {
+        const float u = to_float<T>(ch[i].v[e]);
+        const float u2 = u * u;
+        w.v[e] = from_float<T>(fmaf(u, r1, fmaf(u2, r2, fmaf(u2 * u, r3, c3))));
+      }
+      *reinterpret_cast<u32x4*>(o + (size_t)c * E) = w.raw;
+    }
+  }
+}
+
+template <typename T>
+static void poly_norm_launch(const T* z, long z_stride, T* out, long o_stride, const float* coef, int T_, int F, float eps, hipStream_t stream) {
+  constexpr int E = 16 / (int)sizeof(T);
+  const bool vec = F % E == 0 && z_stride % E == 0 && o_stride % E == 0 && ((uintptr_t)z & 15) == 0 && ((uintptr_t)out & 15) == 0;
+  const int chunks = F / E;
+  if (vec && chunks <= 256 * 2)
+    poly_norm_reg_kernel<T, 256, 2><<<T_, 256, 0, stream>>>(z, z_stride, out, o_stride, coef, F, eps);
+  else if (vec && chunks <= 256 * 4)
+    poly_norm_reg_kernel<T, 256, 4><<<T_, 256, 0, stream>>>(z, z_stride, out, o_stride, coef, F, eps);
+  else if (vec && chunks <= 512 * 8)
+    poly_norm_reg_kernel<T, 512, 8><<<T_, 512, 0, stream>>>(z, z_stride, out, o_stride, coef, F, eps);
+  else
+    poly_norm_kernel<T, 256><<<T_, 256, 0, stream>>>(z, z_stride, out, o_stride, coef, F, eps);
+}
+
 extern "C" int lev_poly_norm(const void* z, long z_stride, void* out, long o_stride, const float* coef, int T, int F, float eps, int dtype,
                              hipStream_t stream) {
   LEV_REQUIRE(T >= 0 && F > 0 && z_stride >= F && o_stride >= F, "poly_norm: bad sizes T=%d F=%d", T, F);
@@ -172,9 +239,9 @@ extern "C" int lev_poly_norm(const void* z, long z_stride, void* out, long o_str
   LEV_REQUIRE(dtype == LEV_F32 || dtype == LEV_BF16, "poly_norm: unknown dtype %d", dtype);
   if (T == 0) return 0;
   if (dtype == LEV_F32)
-    poly_norm_kernel<float, 256><<<T, 256, 0, stream>>>((const float*)z, z_stride, (float*)out, o_stride, coef, F, eps);
+    poly_norm_launch<float>((const float*)z, z_stride, (float*)out, o_stride, coef, T, F, eps, stream);
   else
-    poly_norm_kernel<bf16_t, 256><<<T, 256, 0, stream>>>((const bf16_t*)z, z_stride, (bf16_t*)out, o_stride, coef, F, eps);
+    poly_norm_launch<bf16_t>((const bf16_t*)z, z_stride, (bf16_t*)out, o_stride, coef, T, F, eps, stream);
   return lev_check_launch("poly_norm");
 }
 
@@ -184,24 +251,24 @@ extern "C" int lev_poly_norm(const void* z, long z_stride, void* out, long o_str
 // query heads mixed by `talk` [H][H]:   a[t][h][:] = gate(t, h) * sum_g talk[h][g] * o[t][g][c(h)][:].
 // talk == null: NV is 1 and the sum is o[t][h][0][:]. gate == null: 1, else sigmoid of the gate's entry.
 template <typename T>
-__global__ void __launch_bounds__(256)
+__global__ void __launch_bounds__(64)
 head_talk_kernel(const float* __restrict__ o, const float* __restrict__ talk, const T* __restrict__ gate, long g_stride,
                  T* __restrict__ a, long a_stride, int H, int KVH, int NV, int VD) {
-  const int t = blockIdx.x;
+  const int t = blockIdx.x, h = blockIdx.y;
   const float* ot = o + (size_t)t * H * NV * VD;
-  const int group = H / KVH;
-  for (int e = threadIdx.x; e < H * VD; e += 256) {
-    const int h = e / VD, d = e % VD;
+  const int c = talk ? h / (H / KVH) : 0;
+  float gv = 1.0f;
+  if (gate) gv = 1.0f / (1.0f + expf(-to_float<T>(gate[(size_t)t * g_stride + h])));
+  for (int d = threadIdx.x; d < VD; d += 64) {
     float s;
     if (talk) {
-      const int c = h / group;
       s = 0.f;
+#pragma unroll 8
       for (int g = 0; g < H; ++g) s = fmaf(talk[h * H + g], ot[((size_t)g * NV + c) * VD + d], s);
     } else {
-      s = ot[(size_t)h * NV * VD + d];
+      s = ot[(size_t)h * VD + d];
     }
-    if (gate) s *= 1.0f / (1.0f + expf(-to_float<T>(gate[(size_t)t * g_stride + h])));
-    a[(size_t)t * a_stride + e] = from_float<T>(s);
+    a[(size_t)t * a_stride + (size_t)h * VD + d] = from_float<T>(s * gv);
   }
 }
 
@@ -209,13 +276,13 @@ extern "C" int lev_head_talk(const float* o, const float* talk, const void* gate
                              int KVH, int NV, int VD, int dtype, hipStream_t stream) {
   LEV_REQUIRE(T >= 0 && H > 0 && KVH > 0 && H % KVH == 0 && VD > 0, "head_talk: bad sizes T=%d heads=%d kv_heads=%d vd=%d", T, H, KVH, VD);
   LEV_REQUIRE(NV == (talk ? KVH : 1), "head_talk: %d outputs per query head; with a mixing matrix there are kv_heads=%d, without it one", NV, KVH);
-  LEV_REQUIRE(a_stride >= (long)H * VD, "head_talk: the output's row stride is too small");
+  LEV_REQUIRE(a_stride >= (long)H * VD && H <= 65535, "head_talk: the output's row stride is too small, or too many heads");
   LEV_REQUIRE(dtype == LEV_F32 || dtype == LEV_BF16, "head_talk: unknown dtype %d", dtype);
   if (T == 0) return 0;
   if (dtype == LEV_F32)
-    head_talk_kernel<float><<<T, 256, 0, stream>>>(o, talk, (const float*)gate, g_stride, (float*)a, a_stride, H, KVH, NV, VD);
+    head_talk_kernel<float><<<dim3(T, H), 64, 0, stream>>>(o, talk, (const float*)gate, g_stride, (float*)a, a_stride, H, KVH, NV, VD);
   else
-    head_talk_kernel<bf16_t><<<T, 256, 0, stream>>>(o, talk, (const bf16_t*)gate, g_stride, (bf16_t*)a, a_stride, H, KVH, NV, VD);
+    head_talk_kernel<bf16_t><<<dim3(T, H), 64, 0, stream>>>(o, talk, (const bf16_t*)gate, g_stride, (bf16_t*)a, a_stride, H, KVH, NV, VD);
   return lev_check_launch("head_talk");
 }
 
@@ -269,24 +336,45 @@ extern "C" int lev_stream_average(float* streams, float* x, const float* w, int 
 template <typename TO, int NT>
 __global__ void __launch_bounds__(NT)
 norm_average_kernel(float* __restrict__ streams, float* __restrict__ x, const float* __restrict__ w, int n, long count,
-                    const float* __restrict__ nw, TO* __restrict__ out, const int* __restrict__ rows, int D, float eps) {
+                    const float* __restrict__ nw, TO* __restrict__ out, const int* __restrict__ rows, int D, float eps, int vec) {
   extern __shared__ __attribute__((aligned(16))) float na_row[];
   __shared__ float red[NT / 64];
   const int r = blockIdx.x;
   const long base = (long)(rows ? rows[r] : r) * D;
   const bool store = rows == nullptr;
   float ss = 0.f;
-  for (int d = threadIdx.x; d < D; d += NT) {
-    const float cur = x[base + d];
-    float s = 0.f;
-    for (int j = 0; j < n - 1; ++j) s = fmaf(w[j], streams[(size_t)j * count + base + d], s);
-    s = fmaf(w[n - 1], cur, s);
-    if (store) {
-      streams[(size_t)(n - 1) * count + base + d] = cur;
-      x[base + d] = s;
+  if (vec) {  // D a multiple of 4, every stream 16-byte aligned
+    for (int d = threadIdx.x * 4; d < D; d += NT * 4) {
+      const float4 cur = *reinterpret_cast<const float4*>(x + base + d);
+      float4 s = make_float4(0.f, 0.f, 0.f, 0.f);
+#pragma unroll 4
+      for (int j = 0; j < n - 1; ++j) {
+        const float wj = w[j];
+        const float4 v = *reinterpret_cast<const float4*>(streams + (size_t)j * count + base + d);
+        s.x = fmaf(wj, v.x, s.x); s.y = fmaf(wj, v.y, s.y); s.z = fmaf(wj, v.z, s.z); s.w = fmaf(wj, v.w, s.w);
+      }
+      const float wl = w[n - 1];
+      s.x = fmaf(wl, cur.x, s.x); s.y = fmaf(wl, cur.y, s.y); s.z = fmaf(wl, cur.z, s.z); s.w = fmaf(wl, cur.w, s.w);
+      if (store) {
+        *reinterpret_cast<float4*>(streams + (size_t)(n - 1) * count + base + d) = cur;
+        *reinterpret_cast<float4*>(x + base + d) = s;
+      }
+      *reinterpret_cast<float4*>(na_row + d) = s;
+      ss = fmaf(s.x, s.x, fmaf(s.y, s.y, fmaf(s.z, s.z, fmaf(s.w, s.w, ss))));
     }
-    na_row[d] = s;
-    ss = fmaf(s, s, ss);
+  } else {
+    for (int d = threadIdx.x; d < D; d += NT) {
+      const float cur = x[base + d];
+      float s = 0.f;
+      for (int j = 0; j < n - 1; ++j) s = fmaf(w[j], streams[(size_t)j * count + base + d], s);
+      s = fmaf(w[n - 1], cur, s);
+      if (store) {
+        streams[(size_t)(n - 1) * count + base + d] = cur;
+        x[base + d] = s;
+      }
+      na_row[d] = s;
+      ss = fmaf(s, s, ss);
+    }
   }
   ss = block_sum<NT>(ss, red);
   const float rinv = 1.0f / sqrtf(ss / (float)D + eps);
@@ -301,9 +389,10 @@ extern "C" int lev_norm_average(float* streams, float* x, const float* w, int n,
   LEV_REQUIRE(rows || (long)n_rows * D == count, "norm_average: without a selection every row is normalised");
   if (n_rows == 0) return 0;
   const size_t lds = (size_t)D * sizeof(float);
+  const int vec = D % 4 == 0 && (((uintptr_t)x | (uintptr_t)streams) & 15) == 0;
   if (out_dtype == LEV_F32)
-    norm_average_kernel<float, 256><<<n_rows, 256, lds, stream>>>(streams, x, w, n, count, norm_weight, (float*)out, rows, D, eps);
+    norm_average_kernel<float, 256><<<n_rows, 256, lds, stream>>>(streams, x, w, n, count, norm_weight, (float*)out, rows, D, eps, vec);
   else
-    norm_average_kernel<bf16_t, 256><<<n_rows, 256, lds, stream>>>(streams, x, w, n, count, norm_weight, (bf16_t*)out, rows, D, eps);
+    norm_average_kernel<bf16_t, 256><<<n_rows, 256, lds, stream>>>(streams, x, w, n, count, norm_weight, (bf16_t*)out, rows, D, eps, vec);
   return lev_check_launch("norm_average");
 }

@@ -484,11 +484,27 @@ class HipKernels:
         if dt == torch.bfloat16 and self.use_mfma and self.mfma_attention_values_supports(head_dim, value_dim):
             # matrix cores: runs of several tokens in tiles of 16 query rows, single tokens with the heads of a key/value head as columns
             lib = self._unit(_build.attention_values_unit(head_dim, value_dim))
+            # single tokens: the keys of one token are split over several waves where the step's tokens alone leave the chip
+            # empty (about 1,024 waves are aimed at, a block of 64 keys at least per wave); the step's description keeps the
+            # choice and the scratch memory for all layers with these sizes
+            key = ("values", n_heads, n_kv_heads, value_dim, nv, int(window) if window else 0)
+            plan = meta.plans.get(key)
+            if plan is None:
+                splits = 1
+                if meta.n_decode:
+                    chunks = 1 if nv == 1 else -(-nv * (value_dim // 16) // 16)
+                    reach = min(int(window), meta.max_kv_len) if window else meta.max_kv_len
+                    most = max(1, (reach + 63) // 64 + (1 if window else 0))
+                    splits = int(max(1, min(most, 32, 1024 // max(1, meta.n_decode * n_kv_heads * chunks))))
+                need = lib.lev_attention_values_mfma_workspace(meta.n_decode, splits, n_heads, nv) if splits > 1 else 0
+                ws = torch.empty(need, dtype=torch.uint8, device=q.device) if need else None
+                plan = meta.plans[key] = (splits, ws)
+            splits, ws = plan
             self._check(lib.lev_attention_values_mfma(
                 _ptr(q), _rows(q, "attention_values: q"), _ptr(out), _ptr(k_pages), _ptr(v_pages), _ptr(meta.positions), _ptr(meta.token_seq),
                 _ptr(block_tables), block_tables.shape[1], _ptr(meta.prefill_tiles), meta.n_prefill_tiles, _ptr(meta.decode_tokens),
                 meta.n_decode, n_heads, n_kv_heads, head_dim, value_dim, nv, page_size, float(scale), int(window) if window else 0,
-                float(softcap) if softcap else 0.0, _ptr(slopes), self._s()))
+                float(softcap) if softcap else 0.0, _ptr(slopes), splits, _ptr(ws), self._s()))
             return
         self._check(self.lib.lev_attention_values(
             _ptr(q), _rows(q, "attention_values: q"), _ptr(out), _ptr(k_pages), _ptr(v_pages), _ptr(meta.positions), _ptr(meta.token_seq),
