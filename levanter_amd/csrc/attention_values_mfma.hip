@@ -127,7 +127,8 @@ attention_values_mfma_kernel(const bf16_t* __restrict__ q, long q_stride, float*
 #pragma unroll
     for (int u = 0; u < 2; ++u) {
       const int kp = key0 + 32 * u + 8 * g;
-      pgv[u] = kp <= p_max ? bt[kp / PS] : -1;
+      const int page = bt[min(kp, p_max) / PS];  // loads stand under no condition: a branch would wait for everything in flight
+      pgv[u] = kp <= p_max ? page : -1;
     }
     // scores: S^T tiles (u, h)
     f32x4 st[2][2];
@@ -136,14 +137,14 @@ attention_values_mfma_kernel(const bf16_t* __restrict__ q, long q_stride, float*
 #pragma unroll
       for (int hh = 0; hh < 2; ++hh) {
         const int kp = key0 + 32 * u + 8 * (col >> 2) + 4 * hh + (col & 3);  // the key of this lane's operand row
-        int page = kp <= p_max ? bt[kp / PS] : -1;
-        page = max(page, 0);  // a key without a page is masked below; its operand may be anything that can be read
-        const bf16_t* kb = k_pages + ((size_t)page * KVH + kvh) * k_head + (size_t)(kp % PS) * 8;
+        const int kpc = min(kp, p_max);
+        const int page = max(bt[kpc / PS], 0);  // a key without a page or beyond the range is masked below; its operand may be anything that can be read
+        const bf16_t* kb = k_pages + ((size_t)page * KVH + kvh) * k_head + (size_t)(kpc % PS) * 8;
         f32x4 acc = f32x4{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
         for (int s = 0; s < NKS; ++s) {
           u32x4 kf = u32x4{0u, 0u, 0u, 0u};
-          if (32 * s + 8 * g < HD) kf = *reinterpret_cast<const u32x4*>(kb + (size_t)(4 * s + g) * PS * 8);
+          if (HD % 32 == 0 || 32 * s + 8 * g < HD) kf = *reinterpret_cast<const u32x4*>(kb + (size_t)(4 * s + g) * PS * 8);
           acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_bf16x8(kf), as_bf16x8(qf[s]), acc, 0, 0, 0);
         }
         st[u][hh] = acc;
@@ -239,9 +240,10 @@ attention_values_mfma_kernel(const bf16_t* __restrict__ q, long q_stride, float*
 
 // Runs of several tokens: one workgroup of PF_WAVES waves per (tile of up to PF_ROWS consecutive query tokens, query head,
 // set of value heads). The keys and values of a block of 64 positions are staged once for all waves: global -> registers
-// (requested one block ahead, while the block before is computed) -> LDS, keys as [HD/8][64][8], values transposed as
+// (requested two blocks ahead, while the blocks before are computed) -> LDS, keys as [HD/8][64][8], values transposed as
 // [value head][VD][64 + 8] with everything beyond the last written key made zero on the way.
 #define VS_STRIDE 72
+#define RUN_PAGES 2048  // page ids of a tile's key range that are kept in LDS
 #define K_STAGE ((HD * 8 + PF_THREADS - 1) / PF_THREADS)        // 16-byte chunks of a key block per thread
 #define V_STAGE ((NVC * VD * 8 + PF_THREADS - 1) / PF_THREADS)  // and of the value blocks
 
@@ -253,6 +255,7 @@ attention_values_mfma_runs_kernel(const bf16_t* __restrict__ q, long q_stride, f
   extern __shared__ __attribute__((aligned(16))) unsigned char av_smem[];
   bf16_t* ks = reinterpret_cast<bf16_t*>(av_smem);  // [HD/8][64][8]
   bf16_t* vs = ks + HD * 64;                        // [n_c][VD][VS_STRIDE]
+  __shared__ int pages_s[RUN_PAGES];                // page ids of the blocks that the tile's keys lie in
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, col = lane & 15, g = lane >> 4;
   const int first = tiles[2 * blockIdx.x], n = tiles[2 * blockIdx.x + 1];
   if (n <= 0) return;  // the whole workgroup
@@ -270,6 +273,16 @@ attention_values_mfma_runs_kernel(const bf16_t* __restrict__ q, long q_stride, f
   const float slope = slopes ? slopes[head] : 0.f;
   const int c0 = NV == 1 ? kvh : blockIdx.z * NVC;
   const int n_c = NV == 1 ? 1 : min(NVC, NV - blockIdx.z * NVC);
+  const int key_begin = (lo_wg / 64) * 64;
+  // A key's page: from LDS, where the page ids of the tile's whole key range were put once (a look-up in global memory ahead
+  // of every operand load would put two memory latencies in a row into every block). Pages are powers of two in practice:
+  // a shift then, a division otherwise.
+  const int sh = (PS & (PS - 1)) == 0 ? __builtin_ctz(PS) : -1;
+  const int pg0 = sh >= 0 ? key_begin >> sh : key_begin / PS;
+  const int n_pg = (sh >= 0 ? p_max_wg >> sh : p_max_wg / PS) - pg0 + 1;
+  for (int i = tid; i < min(n_pg, RUN_PAGES); i += PF_THREADS) pages_s[i] = bt[pg0 + i];  // the host sends longer ranges elsewhere
+  auto block_of = [&](int kp) { return sh >= 0 ? kp >> sh : kp / PS; };
+  auto page_of = [&](int kp) { return pages_s[block_of(kp) - pg0]; };  // kp within the tile's range
 
   u32x4 qf[NKS];
 #pragma unroll
@@ -286,35 +299,35 @@ attention_values_mfma_runs_kernel(const bf16_t* __restrict__ q, long q_stride, f
   float m = -INFINITY, l = 0.f;
   constexpr float LOG2E = 1.4426950408889634f;
   const size_t k_head = (size_t)HD * PS, v_head = (size_t)VD * PS;
+  __syncthreads();  // the page ids are there
 
-  u32x4 kst[K_STAGE], vst[V_STAGE];
+  u32x4 kst_a[K_STAGE], vst_a[V_STAGE], kst_b[K_STAGE], vst_b[V_STAGE];  // two blocks on their way at any time
   // this thread's chunks of the block at key0, from the pages into registers
-  auto fetch = [&](int key0) {
+  // Every load stands under no condition (a load in a branch makes the compiler wait for all loads in flight where the
+  // branch ends): addresses are clamped into what can be read, what must not count is made zero afterwards.
+  auto fetch = [&](int key0, u32x4* kst, u32x4* vst) {
 #pragma unroll
     for (int i = 0; i < K_STAGE; ++i) {
-      const int ci = tid + PF_THREADS * i;  // (chunk of 8 dims, key)
-      kst[i] = u32x4{0u, 0u, 0u, 0u};
-      if (ci < HD * 8) {
-        const int kp = key0 + (ci & 63);
-        const int page = kp <= p_max_wg ? bt[kp / PS] : -1;
-        if (page >= 0) kst[i] = *reinterpret_cast<const u32x4*>(k_pages + ((size_t)page * KVH + kvh) * k_head + ((size_t)(ci >> 6) * PS + kp % PS) * 8);
-      }
+      const int ci = min(tid + PF_THREADS * i, HD * 8 - 1);  // (chunk of 8 dims, key)
+      const int kp = key0 + (ci & 63), kpc = min(kp, p_max_wg);
+      const int page = page_of(kpc);
+      const u32x4 v = *reinterpret_cast<const u32x4*>(k_pages + ((size_t)max(page, 0) * KVH + kvh) * k_head +
+                                                      ((size_t)(ci >> 6) * PS + (kpc - block_of(kpc) * PS)) * 8);
+      const uint32_t keep = (kp <= p_max_wg && page >= 0) ? 0xffffffffu : 0u;
+      kst[i] = u32x4{v[0] & keep, v[1] & keep, v[2] & keep, v[3] & keep};
     }
 #pragma unroll
     for (int i = 0; i < V_STAGE; ++i) {
-      const int ci = tid + PF_THREADS * i;  // (value head, dim, group of 8 keys)
-      vst[i] = u32x4{0u, 0u, 0u, 0u};
-      if (ci < n_c * VD * 8) {
-        const int kp = key0 + 8 * (ci & 7), row = ci >> 3;  // row = c * VD + dim
-        const int page = kp <= p_max_wg ? bt[kp / PS] : -1;
-        if (page >= 0) {
-          const u32x4 v = *reinterpret_cast<const u32x4*>(v_pages + ((size_t)page * KVH + c0 + row / VD) * v_head + (size_t)(row % VD) * PS + kp % PS);
-          vst[i] = first_keys(v, min(8, p_max_wg - kp + 1));
-        }
-      }
+      const int ci = min(tid + PF_THREADS * i, n_c * VD * 8 - 1);  // (value head, dim, group of 8 keys)
+      const int kp = key0 + 8 * (ci & 7), row = ci >> 3;         // row = c * VD + dim
+      const int kpc = min(kp, p_max_wg & ~7);
+      const int page = page_of(kpc);
+      const u32x4 v = *reinterpret_cast<const u32x4*>(v_pages + ((size_t)max(page, 0) * KVH + c0 + row / VD) * v_head +
+                                                      (size_t)(row % VD) * PS + (kpc - block_of(kpc) * PS));
+      vst[i] = first_keys(v, page >= 0 ? min(8, max(0, p_max_wg - kp + 1)) : 0);
     }
   };
-  auto stage = [&]() {
+  auto stage = [&](const u32x4* kst, const u32x4* vst) {
 #pragma unroll
     for (int i = 0; i < K_STAGE; ++i) {
       const int ci = tid + PF_THREADS * i;
@@ -327,19 +340,28 @@ attention_values_mfma_runs_kernel(const bf16_t* __restrict__ q, long q_stride, f
     }
   };
 
-  const int key_begin = (lo_wg / 64) * 64;
-  fetch(key_begin);
-  for (int key0 = key_begin; key0 <= p_max_wg; key0 += 64) {
-    __syncthreads();  // the block before has been read by every wave
-    stage();
-    __syncthreads();
-    if (key0 + 64 <= p_max_wg) fetch(key0 + 64);
+  fetch(key_begin, kst_a, vst_a);
+  if (key_begin + 64 <= p_max_wg) fetch(key_begin + 64, kst_b, vst_b);
+  for (int key0 = key_begin, it = 0; key0 <= p_max_wg; key0 += 64, ++it) {
+    lds_barrier();  // the block before has been read by every wave (a barrier for LDS only: the loads on their way stay there)
+    // the register sets take turns: this block's goes to LDS and is asked for again two blocks ahead (conditions uniform
+    // over the workgroup)
+    if (it & 1) {
+      stage(kst_b, vst_b);
+      lds_barrier();
+      if (key0 + 128 <= p_max_wg) fetch(key0 + 128, kst_b, vst_b);
+    } else {
+      stage(kst_a, vst_a);
+      lds_barrier();
+      if (key0 + 128 <= p_max_wg) fetch(key0 + 128, kst_a, vst_a);
+    }
     if (!active || key0 > p_max || key0 + 63 < lo_min) continue;  // none of this wave's rows sees a key of this block
     int pgv[2];
 #pragma unroll
     for (int u = 0; u < 2; ++u) {
       const int kp = key0 + 32 * u + 8 * g;
-      pgv[u] = kp <= p_max ? bt[kp / PS] : -1;
+      const int page = page_of(min(kp, p_max_wg));
+      pgv[u] = kp <= p_max ? page : -1;
     }
     f32x4 st[2][2];
 #pragma unroll
@@ -351,7 +373,7 @@ attention_values_mfma_runs_kernel(const bf16_t* __restrict__ q, long q_stride, f
 #pragma unroll
         for (int s = 0; s < NKS; ++s) {
           u32x4 kf = u32x4{0u, 0u, 0u, 0u};
-          if (32 * s + 8 * g < HD) kf = *reinterpret_cast<const u32x4*>(ks + ((size_t)(4 * s + g) * 64 + key_row) * 8);
+          if (HD % 32 == 0 || 32 * s + 8 * g < HD) kf = *reinterpret_cast<const u32x4*>(ks + ((size_t)(4 * s + g) * 64 + key_row) * 8);
           acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_bf16x8(kf), as_bf16x8(qf[s]), acc, 0, 0, 0);
         }
         st[u][hh] = acc;
@@ -425,30 +447,31 @@ attention_values_mfma_runs_kernel(const bf16_t* __restrict__ q, long q_stride, f
 }
 
 // Merges the splits of a single token's keys: out[tok][head] = sum_s 2^(m_s - M) o_s / sum_s 2^(m_s - M) l_s, in the order of s.
+#define MERGE_MAX_SPLITS 32
 __global__ void __launch_bounds__(64)
 attention_values_merge_kernel(const float* __restrict__ part_o, const float* __restrict__ part_ml, const int* __restrict__ singles,
                               float* __restrict__ out, int H, int n_out, int splits) {
+  __shared__ float w_s[MERGE_MAX_SPLITS + 8];
   const int idx = blockIdx.x, head = blockIdx.y, lane = threadIdx.x;
-  // lane s holds split s's maximum and sum (at most 64 splits)
-  float ms = -INFINITY, ls = 0.f;
-  if (lane < splits) {
-    const size_t slot = ((size_t)idx * splits + lane) * H + head;
-    ms = part_ml[2 * slot];
-    ls = part_ml[2 * slot + 1];
-  }
+  // lane s holds split s's maximum and sum; loads stand under no condition (clamped index, the value replaced afterwards)
+  const float* ml = part_ml + 2 * (((size_t)idx * splits + min(lane, splits - 1)) * H + head);
+  const float mv = ml[0], lv = ml[1];
+  const float ms = lane < splits ? mv : -INFINITY;
   const float M = wave_max(ms);
-  const float ws = __builtin_amdgcn_exp2f(ms - (M == -INFINITY ? 0.f : M));  // no keys: 0
-  float L = ws * ls;
-  // the sum in the order of the splits
-  float Lsum = 0.f;
-  for (int s = 0; s < splits; ++s) Lsum += __shfl(L, s, 64);
-  const float inv = Lsum > 0.f ? 1.0f / Lsum : 0.f;
+  const float w = __builtin_amdgcn_exp2f(ms - (M == -INFINITY ? 0.f : M));  // a split without keys, a lane without a split: 0
+  const float L = wave_sum(w * (lane < splits ? lv : 0.f));
+  if (lane < MERGE_MAX_SPLITS + 8) w_s[lane] = w;
+  __syncthreads();
+  const float inv = L > 0.f ? 1.0f / L : 0.f;
   float* o = out + ((size_t)singles[idx] * H + head) * n_out;
   const float* po = part_o + ((size_t)idx * splits * H + head) * n_out;
   for (int e = lane; e < n_out; e += 64) {
     float acc = 0.f;
-#pragma unroll 4
-    for (int s = 0; s < splits; ++s) acc = fmaf(__shfl(ws, s, 64), po[(size_t)s * H * n_out + e], acc);
+    for (int s0 = 0; s0 < splits; s0 += 8) {
+#pragma unroll
+      for (int j = 0; j < 8; ++j)  // lanes beyond the splits hold weight 0: what they read twice does not count
+        acc = fmaf(w_s[s0 + j], po[(size_t)min(s0 + j, splits - 1) * H * n_out + e], acc);
+    }
     o[e] = acc * inv;
   }
 }
@@ -462,13 +485,14 @@ extern "C" int lev_attention_values_mfma(const void* q, long q_stride, float* ou
                                          const int* positions, const int* token_seq, const int* block_tables, int bt_stride,
                                          const int* tiles, int n_tiles, const int* singles, int n_singles, int H, int KVH, int HD_,
                                          int VD_, int NV, int PS, float scale, int window, float softcap, const float* slopes,
-                                         int splits, float* workspace, hipStream_t stream) {
+                                         int splits, float* workspace, int max_keys, hipStream_t stream) {
   LEV_REQUIRE(HD_ == HD && VD_ == VD, "attention: this library was built for head sizes %d / %d, not %d / %d", HD, VD, HD_, VD_);
   LEV_REQUIRE(H > 0 && KVH > 0 && H % KVH == 0, "attention: bad head counts heads=%d kv_heads=%d", H, KVH);
   LEV_REQUIRE(NV == 1 || NV == KVH, "attention: %d value heads per query head (1 or kv_heads=%d)", NV, KVH);
   LEV_REQUIRE(PS > 0 && PS % 16 == 0, "attention: page_size=%d must be a multiple of 16", PS);
   LEV_REQUIRE(window >= 0 && softcap >= 0.f, "attention: window=%d and soft cap %g must not be negative", window, (double)softcap);
-  LEV_REQUIRE(splits >= 1 && splits <= 64 && (splits == 1 || workspace), "attention: %d splits (at most 64) need scratch memory", splits);
+  LEV_REQUIRE(splits >= 1 && splits <= MERGE_MAX_SPLITS && (splits == 1 || workspace), "attention: %d splits (at most %d) need scratch memory", splits,
+              MERGE_MAX_SPLITS);
   LEV_REQUIRE(n_tiles >= 0 && n_singles >= 0 && (n_tiles == 0 || tiles) && (n_singles == 0 || singles), "attention: bad work lists");
   LEV_REQUIRE(((uintptr_t)q & 15) == 0 && q_stride % 8 == 0 && ((uintptr_t)k_pages & 15) == 0 && ((uintptr_t)v_pages & 15) == 0 &&
                   ((uintptr_t)out & 15) == 0,
@@ -478,11 +502,13 @@ extern "C" int lev_attention_values_mfma(const void* q, long q_stride, float* ou
   if (n_tiles > 0) {
     dim3 grid(n_tiles, H, chunks);
     const size_t lds = ((size_t)HD * 64 + (size_t)(NV == 1 ? 1 : (NV < NVC ? NV : NVC)) * VD * VS_STRIDE) * sizeof(bf16_t);
-    if (lds <= 64 * 1024)
+    // the page ids of a tile's key range (the window, or all keys so far, and the tile itself) must fit their LDS table
+    const long reach = (window > 0 && window < max_keys ? window : max_keys) + PF_ROWS + 64;
+    if (lds + RUN_PAGES * sizeof(int) <= 64 * 1024 && reach / PS + 2 <= RUN_PAGES)
       attention_values_mfma_runs_kernel<<<grid, PF_THREADS, lds, stream>>>((const bf16_t*)q, q_stride, out, (const bf16_t*)k_pages,
                                                                          (const bf16_t*)v_pages, positions, token_seq, block_tables,
                                                                          bt_stride, tiles, H, KVH, NV, PS, scale, window, softcap, slopes);
-    else  // the largest head sizes: every wave by itself, operands straight from the pages
+    else  // the largest head sizes, the longest ranges: every wave by itself, operands straight from the pages
       attention_values_mfma_kernel<false><<<dim3(n_tiles * SUB_TILES, H, chunks), 64, 0, stream>>>(
           (const bf16_t*)q, q_stride, out, (const bf16_t*)k_pages, (const bf16_t*)v_pages, positions, token_seq, block_tables, bt_stride,
           tiles, H, KVH, NV, PS, scale, window, softcap, slopes, 1, nullptr, nullptr);

@@ -181,8 +181,10 @@ poly_norm_reg_kernel(const T* z, long z_stride, T* out, long o_stride, const flo
 #pragma unroll
   for (int i = 0; i < NCH; ++i) {
     const int c = threadIdx.x + NT * i;
-    ch[i].raw = u32x4{0u, 0u, 0u, 0u};
-    if (c < n_chunks) ch[i].raw = *reinterpret_cast<const u32x4*>(row + (size_t)c * E);
+    // under no condition (a load in a branch waits for all loads in flight where the branch ends): clamped, then made zero
+    const u32x4 v = *reinterpret_cast<const u32x4*>(row + (size_t)min(c, n_chunks - 1) * E);
+    const uint32_t keep = c < n_chunks ? 0xffffffffu : 0u;
+    ch[i].raw = u32x4{v[0] & keep, v[1] & keep, v[2] & keep, v[3] & keep};
   }
   float s2 = 0.f, s4 = 0.f, s6 = 0.f;
 #pragma unroll

@@ -92,7 +92,7 @@ def attention_values_unit(head_dim: int, value_dim: int) -> str:
         if head_dim % 16 or value_dim % 16 or not (16 <= head_dim <= 256 and 16 <= value_dim <= 256):
             raise ValueError(f"no matrix-core attention for head sizes {head_dim} / {value_dim}")
         register_unit(name, [("attention_values_mfma.hip", [f"-DLEV_HD={head_dim}", f"-DLEV_VD={value_dim}"], f"attention_values_mfma_hd{head_dim}_vd{value_dim}.o")],
-                      signatures={"lev_attention_values_mfma": [_P, _L, _P, _P, _P, _P, _P, _P, _I, _P, _I, _P, _I] + [_I] * 6 + [_F, _I, _F, _P, _I, _P, _P],
+                      signatures={"lev_attention_values_mfma": [_P, _L, _P, _P, _P, _P, _P, _P, _I, _P, _I, _P, _I] + [_I] * 6 + [_F, _I, _F, _P, _I, _P, _I, _P],
                                   "lev_attention_values_mfma_workspace": [_I, _I, _I, _I]})
     return name
 

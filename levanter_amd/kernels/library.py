@@ -504,7 +504,7 @@ class HipKernels:
                 _ptr(q), _rows(q, "attention_values: q"), _ptr(out), _ptr(k_pages), _ptr(v_pages), _ptr(meta.positions), _ptr(meta.token_seq),
                 _ptr(block_tables), block_tables.shape[1], _ptr(meta.prefill_tiles), meta.n_prefill_tiles, _ptr(meta.decode_tokens),
                 meta.n_decode, n_heads, n_kv_heads, head_dim, value_dim, nv, page_size, float(scale), int(window) if window else 0,
-                float(softcap) if softcap else 0.0, _ptr(slopes), splits, _ptr(ws), self._s()))
+                float(softcap) if softcap else 0.0, _ptr(slopes), splits, _ptr(ws), int(meta.max_kv_len), self._s()))
             return
         self._check(self.lib.lev_attention_values(
             _ptr(q), _rows(q, "attention_values: q"), _ptr(out), _ptr(k_pages), _ptr(v_pages), _ptr(meta.positions), _ptr(meta.token_seq),
