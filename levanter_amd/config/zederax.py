@@ -44,6 +44,8 @@ class ZederaxConfig(LmConfig):
             m = layer.get("mixer")
             if not isinstance(m, dict):
                 raise ConfigError(f"zederax: layer {i} has no 'mixer' sizes")
+            m.setdefault("kv_heads", m.get("heads"))  # left out: every head has keys and values of its own, of one size
+            m.setdefault("vdim", m.get("dim"))
             for key in ("heads", "kv_heads", "dim", "vdim"):
                 if not _positive_int(m.get(key)):
                     raise ConfigError(f"zederax: layer {i}: mixer.{key} must be a positive integer, got {m.get(key)!r}")

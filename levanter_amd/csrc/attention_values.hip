@@ -34,7 +34,11 @@ attention_values_kernel(const T* __restrict__ q, long q_stride, float* __restric
   for (int d = lane; d < HD; d += 64) qs[d] = to_float<T>(q[(size_t)t * q_stride + (size_t)h * HD + d]);
   const float slope = slopes ? slopes[h] : 0.f;
   const int first = window > 0 ? max(0, pos - window + 1) : 0;
-  const int n_out = NV * VD;
+  // more outputs than a lane has accumulators for: blockIdx.z takes the value heads in sets of `heads_per_wave` (the scores
+  // are then computed once per set)
+  const int heads_per_wave = NV == 1 ? 1 : max(1, (64 * AV_MAX_ACC) / VD);
+  const int c_first = NV == 1 ? 0 : blockIdx.z * heads_per_wave;
+  const int n_out = (NV == 1 ? 1 : min(heads_per_wave, NV - c_first)) * VD;
   float acc[AV_MAX_ACC];
 #pragma unroll
   for (int i = 0; i < AV_MAX_ACC; ++i) acc[i] = 0.f;
@@ -70,7 +74,7 @@ attention_values_kernel(const T* __restrict__ q, long q_stride, float* __restric
     for (int i = 0; i < AV_MAX_ACC; ++i) {
       const int e = lane + 64 * i;
       if (e < n_out) {
-        const int c = NV == 1 ? kvh : e / VD, d = e % VD;
+        const int c = NV == 1 ? kvh : c_first + e / VD, d = e % VD;
         float a = acc[i] * corr;
         for (int j = 0; j < n_live; ++j) {
           const int pj = pg[j];
@@ -85,7 +89,7 @@ attention_values_kernel(const T* __restrict__ q, long q_stride, float* __restric
     __syncthreads();
   }
   const float inv = l > 0.f ? 1.0f / l : 0.f;
-  float* o = out + ((size_t)t * H + h) * n_out;
+  float* o = out + ((size_t)t * H + h) * NV * VD + (size_t)c_first * VD;
 #pragma unroll
   for (int i = 0; i < AV_MAX_ACC; ++i) {
     const int e = lane + 64 * i;
@@ -100,14 +104,14 @@ extern "C" int lev_attention_values(const void* q, long q_stride, float* out, co
   LEV_REQUIRE(T >= 0 && H > 0 && KVH > 0 && H % KVH == 0, "attention: bad head counts heads=%d kv_heads=%d", H, KVH);
   LEV_REQUIRE(HD > 0 && HD % 8 == 0 && HD <= AV_MAX_HD, "attention: head_dim=%d must be a multiple of 8 and at most %d", HD, AV_MAX_HD);
   LEV_REQUIRE(VD > 0 && (NV == 1 || NV == KVH), "attention: value size %d, value heads per query head %d (1 or kv_heads=%d)", VD, NV, KVH);
-  LEV_REQUIRE((long)NV * VD <= 64L * AV_MAX_ACC, "attention: %d value heads of %d exceed the %d outputs a query head may have", NV, VD,
-              64 * AV_MAX_ACC);
+  LEV_REQUIRE(VD <= 64 * AV_MAX_ACC, "attention: a value head of %d exceeds the %d outputs a wave may have", VD, 64 * AV_MAX_ACC);
   LEV_REQUIRE(PS > 0 && PS % 16 == 0, "attention: page_size=%d must be a multiple of 16", PS);
   LEV_REQUIRE(H <= 65535, "attention: too many heads (%d)", H);
   LEV_REQUIRE(window >= 0 && softcap >= 0.f, "attention: window=%d and soft cap %g must not be negative", window, (double)softcap);
   LEV_REQUIRE(dtype == LEV_F32 || dtype == LEV_BF16, "attention: unknown dtype %d", dtype);
   if (T == 0) return 0;
-  dim3 grid(T, H);
+  const int per_wave = NV == 1 ? 1 : (64 * AV_MAX_ACC) / VD;
+  dim3 grid(T, H, NV == 1 ? 1 : (NV + per_wave - 1) / per_wave);
   if (dtype == LEV_F32)
     attention_values_kernel<float><<<grid, 64, 0, stream>>>((const float*)q, q_stride, out, (const float*)k_pages, (const float*)v_pages,
                                                            positions, token_seq, block_tables, bt_stride, H, KVH, HD, VD, NV, PS, scale,

@@ -7,11 +7,12 @@
 
 // ------------------------------------------------------------------------------------------
 // One wave per (token, item). Items 0 .. n_norm-1 are heads of `hd` elements that start at column item * hd of the row
-// (queries, then keys: the two lie side by side): x <- x / sqrt(mean(x^2) + eps), in place. Items n_norm .. are value
-// heads of `vd` elements in `v`: v <- (1 - lambda) v + lambda v_first, in place. Either part may be empty.
+// (queries, then keys: the two lie side by side): x <- x / sqrt(sum(x^2) / norm_dim + eps), in place; norm_dim is hd unless
+// the heads are stored with zeros behind their norm_dim elements (head sizes filled up to what the kernels take). Items
+// n_norm .. are value heads of `vd` elements in `v`: v <- (1 - lambda) v + lambda v_first, in place. Either part may be empty.
 template <typename T>
 __global__ void __launch_bounds__(64)
-head_prepare_kernel(T* __restrict__ qk, long qk_stride, int n_norm, int hd, float eps, T* __restrict__ v, long v_stride,
+head_prepare_kernel(T* __restrict__ qk, long qk_stride, int n_norm, int hd, int norm_dim, float eps, T* __restrict__ v, long v_stride,
                     const T* __restrict__ v_first, long vf_stride, int n_blend, int vd, const float* __restrict__ lambda) {
   const int t = blockIdx.x, item = blockIdx.y, lane = threadIdx.x;
   if (item < n_norm) {
@@ -22,7 +23,7 @@ head_prepare_kernel(T* __restrict__ qk, long qk_stride, int n_norm, int hd, floa
       ss = fmaf(x, x, ss);
     }
     ss = wave_sum(ss);
-    const float r = 1.0f / sqrtf(ss / (float)hd + eps);
+    const float r = 1.0f / sqrtf(ss / (float)norm_dim + eps);
     for (int d = lane; d < hd; d += 64) row[d] = from_float<T>(to_float<T>(row[d]) * r);
   } else {
     const int c = item - n_norm;
@@ -35,20 +36,20 @@ head_prepare_kernel(T* __restrict__ qk, long qk_stride, int n_norm, int hd, floa
   }
 }
 
-extern "C" int lev_head_prepare(void* qk, long qk_stride, int n_norm, int hd, float eps, void* v, long v_stride, const void* v_first,
+extern "C" int lev_head_prepare(void* qk, long qk_stride, int n_norm, int hd, int norm_dim, float eps, void* v, long v_stride, const void* v_first,
                                 long vf_stride, int n_blend, int vd, const float* lambda, int T, int dtype, hipStream_t stream) {
   LEV_REQUIRE(T >= 0 && n_norm >= 0 && n_blend >= 0, "head_prepare: bad counts T=%d heads=%d value heads=%d", T, n_norm, n_blend);
-  LEV_REQUIRE(n_norm == 0 || (qk && hd > 0), "head_prepare: heads to normalise need a tensor and a size");
+  LEV_REQUIRE(n_norm == 0 || (qk && hd > 0 && norm_dim > 0 && norm_dim <= hd), "head_prepare: heads to normalise need a tensor and a size");
   LEV_REQUIRE(n_blend == 0 || (v && v_first && lambda && vd > 0), "head_prepare: values to blend need both tensors, a size and the weight");
   LEV_REQUIRE(dtype == LEV_F32 || dtype == LEV_BF16, "head_prepare: unknown dtype %d", dtype);
   LEV_REQUIRE(n_norm + n_blend <= 65535, "head_prepare: too many heads (%d)", n_norm + n_blend);
   if (T == 0 || n_norm + n_blend == 0) return 0;
   dim3 grid(T, n_norm + n_blend);
   if (dtype == LEV_F32)
-    head_prepare_kernel<float><<<grid, 64, 0, stream>>>((float*)qk, qk_stride, n_norm, hd, eps, (float*)v, v_stride, (const float*)v_first,
+    head_prepare_kernel<float><<<grid, 64, 0, stream>>>((float*)qk, qk_stride, n_norm, hd, norm_dim, eps, (float*)v, v_stride, (const float*)v_first,
                                                        vf_stride, n_blend, vd, lambda);
   else
-    head_prepare_kernel<bf16_t><<<grid, 64, 0, stream>>>((bf16_t*)qk, qk_stride, n_norm, hd, eps, (bf16_t*)v, v_stride,
+    head_prepare_kernel<bf16_t><<<grid, 64, 0, stream>>>((bf16_t*)qk, qk_stride, n_norm, hd, norm_dim, eps, (bf16_t*)v, v_stride,
                                                         (const bf16_t*)v_first, vf_stride, n_blend, vd, lambda);
   return lev_check_launch("head_prepare");
 }
@@ -57,17 +58,19 @@ extern "C" int lev_head_prepare(void* qk, long qk_stride, int n_norm, int hd, fl
 // The same for steps of single tokens, with the write into the cache's pages in the same kernel: one wave per (token,
 // item); items are the H query heads (normalised in place), the G key heads (normalised, written to the key pages
 // [page][G][hd/8][PS][8]) and the G value heads (blended, written to the value pages [page][G][vd][PS]). dest[t] =
-// page * PS + offset, negative for a token that is written nowhere. normalise == 0: queries and keys stay as they are.
+// page * PS + offset, negative for a token that is written nowhere. norm_dim: the divisor of the mean of squares (the head's
+// true size); 0: queries and keys stay as they are.
 template <typename T>
 __global__ void __launch_bounds__(64)
 head_prepare_write_kernel(T* __restrict__ q, long q_stride, int H, const T* __restrict__ k, long k_stride, const T* __restrict__ v,
                           long v_stride, const T* __restrict__ v_first, long vf_stride, const float* __restrict__ lambda, int G, int hd,
-                          int vd, float eps, int normalise, T* __restrict__ k_pages, T* __restrict__ v_pages,
+                          int vd, float eps, int norm_dim, T* __restrict__ k_pages, T* __restrict__ v_pages,
                           const int* __restrict__ dest, int PS) {
   const int t = blockIdx.x, item = blockIdx.y, lane = threadIdx.x;
   if (item < H + G) {
     const bool is_q = item < H;
     const T* row = is_q ? q + (size_t)t * q_stride + (size_t)item * hd : k + (size_t)t * k_stride + (size_t)(item - H) * hd;
+    const bool normalise = norm_dim > 0;
     float r = 1.0f;
     if (normalise) {
       float ss = 0.f;
@@ -76,7 +79,7 @@ head_prepare_write_kernel(T* __restrict__ q, long q_stride, int H, const T* __re
         ss = fmaf(x, x, ss);
       }
       ss = wave_sum(ss);
-      r = 1.0f / sqrtf(ss / (float)hd + eps);
+      r = 1.0f / sqrtf(ss / (float)norm_dim + eps);
     }
     if (is_q) {
       if (normalise) {
@@ -113,11 +116,12 @@ head_prepare_write_kernel(T* __restrict__ q, long q_stride, int H, const T* __re
 
 extern "C" int lev_head_prepare_write(void* q, long q_stride, int H, const void* k, long k_stride, const void* v, long v_stride,
                                       const void* v_first, long vf_stride, const float* lambda, int G, int hd, int vd, float eps,
-                                      int normalise, void* k_pages, void* v_pages, const int* dest, int PS, int T, int dtype,
+                                      int norm_dim, void* k_pages, void* v_pages, const int* dest, int PS, int T, int dtype,
                                       hipStream_t stream) {
   LEV_REQUIRE(T >= 0 && H > 0 && G > 0 && hd > 0 && hd % 8 == 0 && vd > 0, "head_prepare_write: bad sizes T=%d heads=%d/%d sizes=%d/%d", T, H, G, hd, vd);
   LEV_REQUIRE(q && k && v && k_pages && v_pages && dest, "head_prepare_write: a tensor is missing");
   LEV_REQUIRE(!v_first || lambda, "head_prepare_write: values to blend need the weight");
+  LEV_REQUIRE(norm_dim >= 0 && norm_dim <= hd, "head_prepare_write: the norm's divisor %d must lie in 0 .. %d", norm_dim, hd);
   LEV_REQUIRE(PS > 0 && PS % 16 == 0, "head_prepare_write: page_size=%d must be a multiple of 16", PS);
   LEV_REQUIRE(H + 2 * G <= 65535, "head_prepare_write: too many heads (%d)", H + 2 * G);
   LEV_REQUIRE(dtype == LEV_F32 || dtype == LEV_BF16, "head_prepare_write: unknown dtype %d", dtype);
@@ -125,12 +129,12 @@ extern "C" int lev_head_prepare_write(void* q, long q_stride, int H, const void*
   dim3 grid(T, H + 2 * G);
   if (dtype == LEV_F32)
     head_prepare_write_kernel<float><<<grid, 64, 0, stream>>>((float*)q, q_stride, H, (const float*)k, k_stride, (const float*)v, v_stride,
-                                                             (const float*)v_first, vf_stride, lambda, G, hd, vd, eps, normalise,
+                                                             (const float*)v_first, vf_stride, lambda, G, hd, vd, eps, norm_dim,
                                                              (float*)k_pages, (float*)v_pages, dest, PS);
   else
     head_prepare_write_kernel<bf16_t><<<grid, 64, 0, stream>>>((bf16_t*)q, q_stride, H, (const bf16_t*)k, k_stride, (const bf16_t*)v,
                                                               v_stride, (const bf16_t*)v_first, vf_stride, lambda, G, hd, vd, eps,
-                                                              normalise, (bf16_t*)k_pages, (bf16_t*)v_pages, dest, PS);
+                                                              norm_dim, (bf16_t*)k_pages, (bf16_t*)v_pages, dest, PS);
   return lev_check_launch("head_prepare_write");
 }
 

@@ -378,9 +378,10 @@ class HipKernels:
 
     # ---- row-wise steps of layers that are not GPT-2's -----------------------------------------
     def head_prepare(self, qk, n_norm: int, head_dim: int, eps: float, v=None, v_first=None, n_blend: int = 0, value_dim: int = 0,
-                     blend=None) -> None:
+                     blend=None, norm_dim: Optional[int] = None) -> None:
         """In place: the ``n_norm`` heads of ``head_dim`` columns at the start of ``qk``'s rows are divided by their root
-        mean square (``sqrt(mean(x^2) + eps)``); the ``n_blend`` heads of ``value_dim`` columns of ``v`` become
+        mean square (``sqrt(sum(x^2) / norm_dim + eps)``; ``norm_dim`` is ``head_dim`` unless the heads carry zeros behind
+        their true size); the ``n_blend`` heads of ``value_dim`` columns of ``v`` become
         ``(1 - blend) v + blend v_first`` (``blend``: a float32 tensor of one element on the GPU). 32-bit arithmetic."""
         T = (qk if qk is not None else v).shape[0]
         dt = (qk if qk is not None else v).dtype
@@ -395,12 +396,12 @@ class HipKernels:
             _req(v.shape == v_first.shape == (T, n_blend * value_dim) and v.dtype == v_first.dtype == dt, "head_prepare: values must be [T, heads*value_dim]")
             _req(blend.dtype == torch.float32 and blend.numel() == 1, "head_prepare: the blending weight must be one float32")
             vs, fs = _rows(v, "head_prepare: v"), _rows(v_first, "head_prepare: v_first")
-        self._check(self.lib.lev_head_prepare(_ptr(qk) if n_norm else None, qs, int(n_norm), int(head_dim), float(eps), _ptr(v) if n_blend else None,
+        self._check(self.lib.lev_head_prepare(_ptr(qk) if n_norm else None, qs, int(n_norm), int(head_dim), int(norm_dim or head_dim), float(eps), _ptr(v) if n_blend else None,
                                               vs, _ptr(v_first) if n_blend else None, fs, int(n_blend), int(value_dim),
                                               _ptr(blend) if n_blend else None, T, _DT[dt], self._s()))
 
     def head_prepare_write(self, q, k, v, k_pages, v_pages, dest, n_heads: int, n_kv_heads: int, head_dim: int, value_dim: int,
-                           page_size: int, eps: Optional[float], v_first=None, blend=None) -> None:
+                           page_size: int, eps: Optional[float], v_first=None, blend=None, norm_dim: Optional[int] = None) -> None:
         """``head_prepare`` and ``kv_write`` in one kernel, for steps of single tokens: queries are normalised in place
         (``eps`` None: not at all), keys are normalised and values blended (``v_first`` None: not) on their way into the pages;
         ``k`` and ``v`` themselves stay as projected."""
@@ -421,7 +422,7 @@ class HipKernels:
         self._check(self.lib.lev_head_prepare_write(
             _ptr(q), _rows(q, "head_prepare_write: q"), n_heads, _ptr(k), _rows(k, "head_prepare_write: k"), _ptr(v),
             _rows(v, "head_prepare_write: v"), _ptr(v_first), fs, _ptr(blend) if v_first is not None else None, n_kv_heads, head_dim,
-            value_dim, float(eps or 0.0), int(eps is not None), _ptr(k_pages), _ptr(v_pages), _ptr(dest), page_size, T, _DT[dt], self._s()))
+            value_dim, float(eps or 0.0), int(norm_dim or head_dim) if eps is not None else 0, _ptr(k_pages), _ptr(v_pages), _ptr(dest), page_size, T, _DT[dt], self._s()))
 
     def poly_norm(self, z, coefficients, eps: float, out) -> None:
         """out = c0 z/rms(z) + c1 z^2/rms(z^2) + c2 z^3/rms(z^3) + c3 per row, rms(u) = sqrt(mean(u^2) + eps); powers element

@@ -51,7 +51,7 @@ def zederax_model_spec(cfg: ZederaxConfig) -> ModelSpec:
             "talk": TensorSpec(f"{p}.mix.talk", (H, H), init="eye_plus_normal", std=0.3),
             "out.weight": TensorSpec(f"{p}.mix.o", (d, H * vd), std=1.0 / math.sqrt(H * vd)),
         }
-        if m.get("v_mix"):  # the first blending layer's weight is stored too and not used
+        if value_mix == "blend":  # the source layer's own weight may be stored too; it is not used (see ignored_tensors)
             tensors["value_mix.weight"] = TensorSpec(f"{p}.mix.vmix", (), init="unit_interval")
         mixer = PartSpec(
             "talking_heads_attention",
@@ -85,5 +85,7 @@ def zederax_model_spec(cfg: ZederaxConfig) -> ModelSpec:
         final_norm=rms_norm("final.norm"),
         head=head,
         max_positions=None,
+        # a blend weight that a file stores for a layer that does not blend (the values' source, a layer without the blend)
+        ignored_tensors=(r"l\d+\.mix\.vmix",),
         init_std=cfg.initializer_range,
     )

@@ -67,8 +67,14 @@ class ParallelBlock(Block):
             dev = (a if a is not None else b).device
             return torch.cat([a if a is not None else torch.zeros(na, device=dev), b if b is not None else torch.zeros(nb, device=dev)])
 
-        self.n_mixer_cols, self.n_mixer_heads = m.proj.n_out, m.out.n_in
-        self.fused_in = Linear(torch.cat([m.proj.weight, f.up.weight], 0), cat_bias(m.proj.bias, f.up.bias, m.proj.n_out, f.up.n_out), "out_in", env)
+        self.n_mixer_cols, self.n_mixer_heads, self.n_inner = m.proj.n_out, m.out.n_in, f.up.n_out
+        # rows of zeros at the end keep the product's rows a multiple of 8 wide, so that 16-byte loads of the heads stay aligned
+        fill = (-(m.proj.n_out + f.up.n_out)) % 8
+        w_in = torch.cat([m.proj.weight, f.up.weight, torch.zeros(fill, m.proj.n_in, dtype=m.proj.weight.dtype, device=m.proj.weight.device)], 0)
+        b_in = cat_bias(m.proj.bias, f.up.bias, m.proj.n_out, f.up.n_out)
+        if b_in is not None and fill:
+            b_in = torch.cat([b_in, torch.zeros(fill, device=b_in.device)])
+        self.fused_in = Linear(w_in, b_in, "out_in", env)
         out_bias = None if m.out.bias is None and f.down.bias is None else sum(b for b in (m.out.bias, f.down.bias) if b is not None)
         self.fused_out = Linear(torch.cat([m.out.weight, f.down.weight], 1), out_bias, "out_in", env)
         m.proj = m.out = f.up = f.down = None
@@ -85,7 +91,7 @@ class ParallelBlock(Block):
             pz = self.fused_in(h, ctx)  # [T, the mixer's projections | the feed-forward's]
             am = ctx.empty(h.shape[0], self.fused_out.n_in)
             self.mixer.attend(pz[:, :self.n_mixer_cols], ctx, unit, writes_cache, am[:, :self.n_mixer_heads])
-            self.feed_forward.activate(pz[:, self.n_mixer_cols:], ctx, am[:, self.n_mixer_heads:])
+            self.feed_forward.activate(pz[:, self.n_mixer_cols:self.n_mixer_cols + self.n_inner], ctx, am[:, self.n_mixer_heads:])
             self.fused_out(am, ctx, residual=x)
         else:
             self.mixer.forward(h, x, ctx, unit, writes_cache)

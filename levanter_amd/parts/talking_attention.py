@@ -54,8 +54,13 @@ class TalkingHeadsAttention(Mixer):
         self.unit_norm_eps = p.get("unit_norm_eps")
         if self.n_heads % self.n_kv_heads != 0:
             raise ValueError(f"attention: {self.n_heads} heads are not a multiple of {self.n_kv_heads} key/value heads")
-        if self.head_dim % 8 != 0 or self.value_dim % 8 != 0:
-            raise ValueError(f"attention: head sizes {self.head_dim} (keys) and {self.value_dim} (values) must be multiples of 8")
+        # The cache keeps keys in chunks of 8 elements and the matrix-core kernels work on tiles of 16: heads of any other
+        # size are stored with zeros behind them (rows of zeros in the projections, columns of zeros in the output
+        # projection). Zeros change no score and no output; only the unit norm has to divide by the true size.
+        step = 16 if env.dtype == torch.bfloat16 else 8
+        self.true_head_dim, self.true_value_dim = self.head_dim, self.value_dim
+        self.head_dim = (self.head_dim + step - 1) // step * step
+        self.value_dim = (self.value_dim + step - 1) // step * step
         slopes = p.get("distance_slopes")
         self.slopes = None
         if slopes is not None:
@@ -78,26 +83,39 @@ class TalkingHeadsAttention(Mixer):
         self.q_cols, self.k_cols, self.v_cols = self.n_heads * self.head_dim, self.n_kv_heads * self.head_dim, self.n_kv_heads * self.value_dim
         names = ["q", "k", "v"] + (["gate"] if "gate.weight" in tensors else [])
         sizes = {"q": self.q_cols, "k": self.k_cols, "v": self.v_cols, "gate": self.n_heads}
+        # (heads, size in the checkpoint, size as stored here) of each projection
+        heads_of = {"q": (self.n_heads, self.true_head_dim, self.head_dim), "k": (self.n_kv_heads, self.true_head_dim, self.head_dim),
+                    "v": (self.n_kv_heads, self.true_value_dim, self.value_dim), "gate": (1, self.n_heads, self.n_heads)}
         rows, biases, self.offsets, at = [], [], {}, 0
         any_bias = any(f"{n}.bias" in tensors for n in names)
         for n in names:
-            w = tensors[f"{n}.weight"].to(torch.float32)
-            if tuple(w.shape) != (sizes[n], self.dim):
-                raise ValueError(f"attention: {n}.weight must be [{sizes[n]}, {self.dim}], got {list(w.shape)}")
+            nh, true, stored = heads_of[n]
+            w = tensors[f"{n}.weight"].to(torch.float32).cpu()
+            if tuple(w.shape) != (nh * true, self.dim):
+                raise ValueError(f"attention: {n}.weight must be [{nh * true}, {self.dim}], got {list(w.shape)}")
             b = tensors.get(f"{n}.bias")
-            b = torch.zeros(sizes[n]) if b is None else b.to(torch.float32).cpu()
+            b = torch.zeros(nh * true) if b is None else b.to(torch.float32).cpu()
+            if stored != true:  # zeros behind every head
+                w = torch.cat([w.view(nh, true, self.dim), torch.zeros(nh, stored - true, self.dim)], 1).reshape(nh * stored, self.dim)
+                b = torch.cat([b.view(nh, true), torch.zeros(nh, stored - true)], 1).reshape(nh * stored)
             pad = _pad8(sizes[n]) - sizes[n]
             self.offsets[n] = at
-            rows += [w.cpu(), torch.zeros(pad, self.dim)]
+            rows += [w, torch.zeros(pad, self.dim)]
             biases += [b, torch.zeros(pad)]
             at += sizes[n] + pad
         if self.offsets["k"] != self.q_cols:
             raise ValueError("attention: heads * head_dim must be a multiple of 8 (keys follow the queries without a gap)")
         self.proj = Linear(torch.cat(rows, 0), torch.cat(biases, 0) if any_bias else None, "out_in", env)
         self.has_gate = "gate" in self.offsets
-        self.out = Linear(tensors["out.weight"], tensors.get("out.bias"), p.get("weight_layout", "out_in"), env)
-        if (self.out.n_in, self.out.n_out) != (self.n_heads * self.value_dim, self.dim):
+        w_out = tensors["out.weight"]
+        if p.get("weight_layout", "out_in") == "in_out":
+            w_out = w_out.t()
+        if tuple(w_out.shape) != (self.dim, self.n_heads * self.true_value_dim):
             raise ValueError("attention: the output projection does not have the sizes of the description")
+        if self.value_dim != self.true_value_dim:  # columns of zeros where the heads carry zeros
+            w_out = torch.cat([w_out.to(torch.float32).cpu().reshape(self.dim, self.n_heads, self.true_value_dim),
+                               torch.zeros(self.dim, self.n_heads, self.value_dim - self.true_value_dim)], 2).reshape(self.dim, -1)
+        self.out = Linear(w_out, tensors.get("out.bias"), "out_in", env)
 
     def cache_requirement(self):
         return PagedKv(self.n_kv_heads, self.head_dim, self.window, None if self.value_dim == self.head_dim else self.value_dim)
@@ -129,12 +147,13 @@ class TalkingHeadsAttention(Mixer):
         if writes_cache and ctx.attention.n_prefill_tiles == 0:
             # a step of single tokens: unit norms, the blend and the write into the pages are one kernel
             K.head_prepare_write(q, k, v, unit.k_pages, unit.v_pages, g.dest, self.n_heads, self.n_kv_heads, self.head_dim, self.value_dim,
-                                 g.page_size, self.unit_norm_eps, v_first=v_first, blend=self.blend)
+                                 g.page_size, self.unit_norm_eps, v_first=v_first, blend=self.blend, norm_dim=self.true_head_dim)
         else:
             n_norm = self.n_heads + self.n_kv_heads if self.unit_norm_eps is not None else 0
             if n_norm or v_first is not None:
                 K.head_prepare(p[:, :self.q_cols + self.k_cols], n_norm, self.head_dim, self.unit_norm_eps or 0.0, v=v, v_first=v_first,
-                               n_blend=self.n_kv_heads if v_first is not None else 0, value_dim=self.value_dim, blend=self.blend)
+                               n_blend=self.n_kv_heads if v_first is not None else 0, value_dim=self.value_dim, blend=self.blend,
+                               norm_dim=self.true_head_dim)
             if writes_cache:  # keys and values of 16 tokens at a time, transposed through LDS
                 K.kv_write(k, v, unit.k_pages, unit.v_pages, g.dest, self.n_kv_heads, self.head_dim, g.page_size, value_dim=self.value_dim)
         nv = self.n_kv_heads if self.talk is not None else 1

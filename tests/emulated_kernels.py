@@ -164,21 +164,21 @@ class EmulatedKernels:
         return False
 
     # ---- row-wise steps of layers that are not GPT-2's
-    def head_prepare(self, qk, n_norm, head_dim, eps, v=None, v_first=None, n_blend=0, value_dim=0, blend=None) -> None:
+    def head_prepare(self, qk, n_norm, head_dim, eps, v=None, v_first=None, n_blend=0, value_dim=0, blend=None, norm_dim=None) -> None:
         if n_norm:
             x = qk[:, :n_norm * head_dim].float().view(qk.shape[0], n_norm, head_dim)
-            x = x / torch.sqrt((x * x).mean(-1, keepdim=True) + eps)
+            x = x / torch.sqrt((x * x).sum(-1, keepdim=True) / (norm_dim or head_dim) + eps)
             qk[:, :n_norm * head_dim] = x.reshape(qk.shape[0], -1).to(qk.dtype)
         if n_blend:
             lam = float(blend.reshape(-1)[0])
             v.copy_(((1.0 - lam) * v.float() + lam * v_first.float()).to(v.dtype))
 
     def head_prepare_write(self, q, k, v, k_pages, v_pages, dest, n_heads, n_kv_heads, head_dim, value_dim, page_size, eps, v_first=None,
-                           blend=None) -> None:
+                           blend=None, norm_dim=None) -> None:
         k, v = k.clone(), v.clone()
         if eps is not None:
-            self.head_prepare(q, n_heads, head_dim, eps)
-            self.head_prepare(k, n_kv_heads, head_dim, eps)
+            self.head_prepare(q, n_heads, head_dim, eps, norm_dim=norm_dim)
+            self.head_prepare(k, n_kv_heads, head_dim, eps, norm_dim=norm_dim)
         if v_first is not None:
             self.head_prepare(None, 0, 0, 0.0, v=v, v_first=v_first, n_blend=n_kv_heads, value_dim=value_dim, blend=blend)
         self.kv_write(k, v, k_pages, v_pages, dest, n_kv_heads, head_dim, page_size, value_dim=value_dim)

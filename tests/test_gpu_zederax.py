@@ -218,6 +218,7 @@ ATT_SHAPES = [  # H, G, dk, dv, window, cap
     (2, 1, 128, 16, 33, 50.0),
     (8, 8, 16, 64, 40, 10.0),   # more value heads than one wave of the matrix-core kernel takes
     (34, 2, 16, 16, 21, 10.0),  # more query heads per key/value head than a wave has columns
+    (6, 6, 8, 408, 30, 10.0),   # more outputs a query head than a wave of the plain kernel holds (and no matrix-core kernel)
 ]
 
 
@@ -299,10 +300,10 @@ def row_error(got, want):
     return (d.pow(2).mean(-1).sqrt() / want.std(-1)).max().item()
 
 
-LENGTHS = {"A": [70, 45, 100, 37, 64, 33], "B": [90, 130, 41, 200, 64, 17], "C": [40, 12, 30, 3]}
+LENGTHS = {"A": [70, 45, 100, 37, 64, 33], "B": [90, 130, 41, 200, 64, 17], "C": [40, 12, 30, 3], "D": [66, 21, 80, 5, 97]}
 
 
-@pytest.mark.parametrize("name", ["A", "B", "C"])
+@pytest.mark.parametrize("name", ["A", "B", "C", "D"])
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 def test_trace_run_all_cuttings(name, dtype, tmp_path):
     """Whole prompts, the last 32 tokens one by one, portions down to two tokens, and twice mixed with other requests in a pool

@@ -27,10 +27,10 @@ def build(name, tmp, dtype=torch.float32):
     return raw, W, model, env, config
 
 
-@pytest.fixture(scope="module", params=["A", "B", "C"])
+@pytest.fixture(scope="module", params=["A", "B", "C", "D"])
 def setup(request, tmp_path_factory):
     raw, W, model, env, _ = build(request.param, tmp_path_factory.mktemp("zed"))
-    lengths = {"A": [70, 45, 100, 37, 64, 33], "B": [90, 130, 41, 17, 64], "C": [40, 12, 30]}[request.param]
+    lengths = {"A": [70, 45, 100, 37, 64, 33], "B": [90, 130, 41, 17, 64], "C": [40, 12, 30], "D": [66, 21, 80, 5]}[request.param]
     reqs = TR.random_requests(raw["vocab"], lengths, 5)
     plain = {rid: Z.plain_logits(W, raw, torch.tensor(t)) for rid, t in reqs.items()}
     return raw, W, model, env, reqs, plain

@@ -24,4 +24,11 @@ ZED_C = Z.make_config(vocab=50, width=32, eps=1e-3, layers=[
     Z.layer(heads=1, kv_heads=1, dim=8, vdim=24, window=9, softcap=2.0, v_mix=True, ff=16),
 ])
 
-ZED = {"A": (ZED_A, 11), "B": (ZED_B, 12), "C": (ZED_C, 13)}
+# head sizes that are no multiple of 8 (the engine stores such heads with zeros behind them), widths that are no multiple of 4
+ZED_D = Z.make_config(vocab=61, width=50, eps=1e-5, layers=[
+    Z.layer(heads=3, kv_heads=1, dim=12, vdim=20, window=19, softcap=6.0, v_mix=True, ff=30),
+    Z.layer(heads=2, kv_heads=2, dim=20, vdim=10, window=None, softcap=None, v_mix=False, ff=33),
+    Z.layer(heads=3, kv_heads=1, dim=36, vdim=20, window=50, softcap=12.0, v_mix=True, ff=None),
+])
+
+ZED = {"A": (ZED_A, 11), "B": (ZED_B, 12), "C": (ZED_C, 13), "D": (ZED_D, 14)}
